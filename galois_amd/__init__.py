@@ -1,0 +1,169 @@
+"""galois_amd -- MI355X (gfx950) backend for galois's Q4_0 quantized-matmul path.
+
+The product is ``libgalois_hip.so`` (hand-written HIP kernels behind the C ABI of
+``include/galois_hip.h``).  This package is the thin Python face of that ABI used by
+the tests and the benchmark: device buffers, copies, events and one method per entry
+point, argument for argument.  There is no CPU fallback: importing works anywhere,
+but creating a :class:`Device` without the built library or without a gfx950 GPU
+raises.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _abi
+
+__all__ = ["Device", "DeviceBuffer", "GaloisHipError", "Q4_0_BLOCK_BYTES", "QK4_0"]
+
+QK4_0 = 32
+Q4_0_BLOCK_BYTES = 18
+
+
+class GaloisHipError(RuntimeError):
+    def __init__(self, status, text):
+        super().__init__("galois_hip status %d: %s" % (status, text))
+        self.status = status
+
+
+class DeviceBuffer:
+    """Owning handle of device memory (the reference's CudaSlice<T>); ``ptr`` is a raw address."""
+
+    def __init__(self, dev, ptr, nbytes, owner=True):
+        self.dev, self.ptr, self.nbytes, self._owner = dev, ptr, nbytes, owner
+
+    def view(self, byte_offset, nbytes=None):
+        """Sub-view by pointer arithmetic (``.slice(offset..)`` in the reference, src/cuda.rs:54-73)."""
+        assert 0 <= byte_offset <= self.nbytes
+        nbytes = self.nbytes - byte_offset if nbytes is None else nbytes
+        assert byte_offset + nbytes <= self.nbytes
+        return DeviceBuffer(self.dev, self.ptr + byte_offset, nbytes, owner=False)
+
+    def free(self):
+        if self._owner and self.ptr:
+            self.dev._check(self.dev._lib.galois_hip_free(self.dev._ctx, self.ptr))
+            self.ptr = 0
+
+    def __int__(self):
+        return self.ptr
+
+
+def _ptr(b):
+    if b is None:
+        return None
+    return C.c_void_p(b.ptr if isinstance(b, DeviceBuffer) else int(b))
+
+
+class Device:
+    """One device ordinal + one stream (``CudaDevice::new``, src/cuda.rs:221-229)."""
+
+    def __init__(self, ordinal=0):
+        self._lib = _abi.load()
+        ctx = C.c_void_p()
+        st = self._lib.galois_hip_create(ordinal, C.byref(ctx))
+        if st != 0:
+            raise GaloisHipError(st, self._lib.galois_hip_status_string(st).decode())
+        self._ctx = ctx
+        self._bufs = []
+        n = C.c_int32()
+        self._check(self._lib.galois_hip_init_functions(self._ctx, 1, C.byref(n)))
+        self.n_kernels = n.value
+
+    # -- plumbing ---------------------------------------------------------------
+    def _check(self, st):
+        if st != 0:
+            raise GaloisHipError(st, self._lib.galois_hip_last_error(self._ctx).decode()
+                                 or self._lib.galois_hip_status_string(st).decode())
+
+    def close(self):
+        if self._ctx:
+            for b in self._bufs:
+                b.free()
+            self._bufs = []
+            self._lib.galois_hip_destroy(self._ctx)
+            self._ctx = None
+
+    def info(self):
+        name, arch = C.create_string_buffer(256), C.create_string_buffer(256)
+        ncu, clk, mclk, mem = C.c_int32(), C.c_int32(), C.c_int32(), C.c_int64()
+        self._check(self._lib.galois_hip_device_info(self._ctx, name, 256, arch, 256, C.byref(ncu), C.byref(clk),
+                                                     C.byref(mclk), C.byref(mem)))
+        return {"name": name.value.decode(), "arch": arch.value.decode(), "n_cu": ncu.value,
+                "clock_khz": clk.value, "mem_clock_khz": mclk.value, "mem_bytes": mem.value}
+
+    def alloc(self, nbytes):
+        p = C.c_void_p()
+        self._check(self._lib.galois_hip_alloc_zeros(self._ctx, nbytes, C.byref(p)))
+        b = DeviceBuffer(self, p.value or 0, nbytes)
+        self._bufs.append(b)
+        return b
+
+    def free(self, buf):
+        buf.free()
+        self._bufs = [b for b in self._bufs if b is not buf]
+
+    def upload(self, arr, buf=None):
+        arr = np.ascontiguousarray(arr)
+        if buf is None:
+            buf = self.alloc(arr.nbytes)
+        assert arr.nbytes <= buf.nbytes
+        self._check(self._lib.galois_hip_htod_sync_copy(self._ctx, _ptr(buf), arr.ctypes.data_as(C.c_void_p),
+                                                        arr.nbytes))
+        return buf
+
+    def download(self, buf, dtype, shape):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= buf.nbytes
+        self._check(self._lib.galois_hip_dtoh_sync_copy(self._ctx, out.ctypes.data_as(C.c_void_p), _ptr(buf),
+                                                        out.nbytes))
+        return out
+
+    def copy_d2d(self, dst, src, nbytes):
+        self._check(self._lib.galois_hip_dtod_copy(self._ctx, _ptr(dst), _ptr(src), nbytes))
+
+    def copy_d2d_2d(self, dst, dpitch, src, spitch, width, height):
+        self._check(self._lib.galois_hip_dtod_copy_2d(self._ctx, _ptr(dst), dpitch, _ptr(src), spitch, width, height))
+
+    def synchronize(self):
+        self._check(self._lib.galois_hip_synchronize(self._ctx))
+
+    def event(self):
+        ev = C.c_void_p()
+        self._check(self._lib.galois_hip_event_create(self._ctx, C.byref(ev)))
+        return ev
+
+    def record(self, ev):
+        self._check(self._lib.galois_hip_event_record(self._ctx, ev))
+
+    def elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        self._check(self._lib.galois_hip_event_elapsed_ms(self._ctx, start, stop, C.byref(ms)))
+        return ms.value
+
+    def event_destroy(self, ev):
+        self._check(self._lib.galois_hip_event_destroy(self._ctx, ev))
+
+    # -- ops: same argument order as the C ABI ----------------------------------------
+    def dequantize_mul_mat_vec_q4_0(self, vx, y, dst, ncols, nrows):
+        self._check(self._lib.galois_hip_dequantize_mul_mat_vec_q4_0(self._ctx, _ptr(vx), _ptr(y), _ptr(dst),
+                                                                     ncols, nrows))
+
+    def mul_mat_q4_0_f32(self, W, X, Y, K, N, M):
+        self._check(self._lib.galois_hip_mul_mat_q4_0_f32(self._ctx, _ptr(W), _ptr(X), _ptr(Y), K, N, M))
+
+    def rms_norm_f32(self, x, dst, ncols, nrows, eps):
+        self._check(self._lib.galois_hip_rms_norm_f32(self._ctx, _ptr(x), _ptr(dst), ncols, nrows, eps))
+
+    def rms_norm_mul_f32(self, x, weight, dst, ncols, nrows, eps):
+        self._check(self._lib.galois_hip_rms_norm_mul_f32(self._ctx, _ptr(x), _ptr(weight), _ptr(dst), ncols, nrows,
+                                                          eps))
+
+    def rope_f32(self, x, dst, ncols, nrows, pos, freq_scale, p_delta_rows, theta_scale):
+        self._check(self._lib.galois_hip_rope_f32(self._ctx, _ptr(x), _ptr(dst), ncols, nrows, _ptr(pos), freq_scale,
+                                                  p_delta_rows, theta_scale))
+
+    def soft_max_f32(self, x, dst, ncols, nrows):
+        self._check(self._lib.galois_hip_soft_max_f32(self._ctx, _ptr(x), _ptr(dst), ncols, nrows))
+
+    def soft_max_causal_f32(self, x, dst, ncols, rows_per_head, nrows, n_past):
+        self._check(self._lib.galois_hip_soft_max_causal_f32(self._ctx, _ptr(x), _ptr(dst), ncols, rows_per_head,
+                                                             nrows, n_past))

@@ -1,0 +1,59 @@
+// Shared internals of libgalois_hip: context object, status helpers, Q4_0 block.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/galois_hip.h"
+
+struct galois_hip_ctx {
+    int32_t ordinal;
+    hipStream_t stream;
+    int32_t n_cu;
+    int32_t gemv_config;  // 0 = choose from the shape; GALOIS_HIP_GEMV_CONFIG=1..5 forces a kernel shape (tuning)
+    char last_error[256];
+};
+
+struct galois_hip_event {
+    hipEvent_t ev;
+};
+
+// Q4_0 block exactly as the reference stores it (src/ggml_quants.rs:140-145).
+struct block_q4_0 {
+    uint16_t d;      // f16 bits
+    uint8_t qs[16];  // weight j = low nibble of qs[j], weight j+16 = high nibble
+};
+static_assert(sizeof(block_q4_0) == 18, "Q4_0 block must be 18 bytes");
+
+static inline int32_t gh_fail(galois_hip_ctx *ctx, int32_t status, const char *what) {
+    if (ctx) snprintf(ctx->last_error, sizeof(ctx->last_error), "%s: %s", what, galois_hip_status_string(status));
+    return status;
+}
+
+static inline int32_t gh_hip(galois_hip_ctx *ctx, hipError_t e, const char *what) {
+    if (e == hipSuccess) return GALOIS_HIP_OK;
+    if (ctx) snprintf(ctx->last_error, sizeof(ctx->last_error), "%s: %s", what, hipGetErrorString(e));
+    return (int32_t)e;
+}
+
+#define GH_REQUIRE_CTX(ctx) \
+    do {                    \
+        if (!(ctx)) return GALOIS_HIP_E_NULL; \
+    } while (0)
+
+#define GH_REQUIRE(ctx, cond, status, what)            \
+    do {                                               \
+        if (!(cond)) return gh_fail((ctx), (status), (what)); \
+    } while (0)
+
+// Binds the context's device to the calling thread, then checks the launch that follows.
+#define GH_BIND(ctx)                                                       \
+    do {                                                                   \
+        hipError_t e__ = hipSetDevice((ctx)->ordinal);                     \
+        if (e__ != hipSuccess) return gh_hip((ctx), e__, "hipSetDevice"); \
+    } while (0)
+
+#define GH_LAUNCH_CHECK(ctx, what) return gh_hip((ctx), hipGetLastError(), (what))
+
+static inline bool gh_aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }

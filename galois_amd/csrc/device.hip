@@ -1,0 +1,198 @@
+// Device / stream / buffer layer of libgalois_hip (replaces what src/cuda.rs:35-308
+// obtains from cudarc).  One context = one device ordinal + one stream.
+#include "common.h"
+
+#include <stdlib.h>
+
+extern "C" {
+
+const char *galois_hip_status_string(int32_t s) {
+    switch (s) {
+        case GALOIS_HIP_OK: return "ok";
+        case GALOIS_HIP_E_NULL: return "null pointer argument";
+        case GALOIS_HIP_E_SHAPE: return "bad shape argument";
+        case GALOIS_HIP_E_ALIGN: return "misaligned device pointer";
+        case GALOIS_HIP_E_ORDINAL: return "no such device";
+        case GALOIS_HIP_E_UNSUPPORTED: return "unsupported combination";
+        case GALOIS_HIP_E_ARCH: return "device is not gfx950";
+        default: return s > 0 ? hipGetErrorString((hipError_t)s) : "unknown status";
+    }
+}
+
+int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
+    if (!out) return GALOIS_HIP_E_NULL;
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) return (int32_t)e;
+    if (ordinal < 0 || ordinal >= n) return GALOIS_HIP_E_ORDINAL;
+    e = hipSetDevice(ordinal);
+    if (e != hipSuccess) return (int32_t)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, ordinal);
+    if (e != hipSuccess) return (int32_t)e;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return GALOIS_HIP_E_ARCH;
+    galois_hip_ctx *ctx = new galois_hip_ctx();
+    ctx->ordinal = ordinal;
+    ctx->n_cu = prop.multiProcessorCount;
+    ctx->last_error[0] = 0;
+    const char *cfg = getenv("GALOIS_HIP_GEMV_CONFIG");
+    ctx->gemv_config = cfg ? atoi(cfg) : 0;
+    e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete ctx;
+        return (int32_t)e;
+    }
+    *out = ctx;
+    return GALOIS_HIP_OK;
+}
+
+int32_t galois_hip_destroy(galois_hip_ctx *ctx) {
+    GH_REQUIRE_CTX(ctx);
+    (void)hipSetDevice(ctx->ordinal);
+    (void)hipStreamSynchronize(ctx->stream);
+    hipError_t e = hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return (int32_t)e;
+}
+
+int32_t galois_hip_init_functions(galois_hip_ctx *ctx, int32_t abi_version, int32_t *n_kernels) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, abi_version == GALOIS_HIP_ABI_VERSION, GALOIS_HIP_E_UNSUPPORTED, "init_functions: ABI version");
+    if (n_kernels) *n_kernels = 16;  // the reference registers 16 kernel names (src/kernels.rs:5-20)
+    return GALOIS_HIP_OK;
+}
+
+const char *galois_hip_last_error(const galois_hip_ctx *ctx) { return ctx ? ctx->last_error : ""; }
+
+int32_t galois_hip_device_info(galois_hip_ctx *ctx, char *name, int32_t name_cap, char *arch, int32_t arch_cap,
+                               int32_t *n_cu, int32_t *clock_khz, int32_t *mem_clock_khz, int64_t *mem_bytes) {
+    GH_REQUIRE_CTX(ctx);
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, ctx->ordinal);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipGetDeviceProperties");
+    if (name && name_cap > 0) snprintf(name, (size_t)name_cap, "%s", prop.name);
+    if (arch && arch_cap > 0) snprintf(arch, (size_t)arch_cap, "%s", prop.gcnArchName);
+    if (n_cu) *n_cu = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    if (mem_clock_khz) *mem_clock_khz = prop.memoryClockRate;
+    if (mem_bytes) *mem_bytes = (int64_t)prop.totalGlobalMem;
+    return GALOIS_HIP_OK;
+}
+
+int32_t galois_hip_alloc_zeros(galois_hip_ctx *ctx, size_t bytes, void **out) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, out != nullptr, GALOIS_HIP_E_NULL, "alloc_zeros: out");
+    *out = nullptr;
+    GH_BIND(ctx);
+    if (bytes == 0) return GALOIS_HIP_OK;  // empty slice: NULL pointer, like an empty CudaSlice
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipMalloc");
+    e = hipMemsetAsync(p, 0, bytes, ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(p);
+        return gh_hip(ctx, e, "hipMemsetAsync");
+    }
+    *out = p;
+    return GALOIS_HIP_OK;
+}
+
+int32_t galois_hip_free(galois_hip_ctx *ctx, void *dptr) {
+    GH_REQUIRE_CTX(ctx);
+    if (!dptr) return GALOIS_HIP_OK;
+    GH_BIND(ctx);
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipStreamSynchronize");
+    return gh_hip(ctx, hipFree(dptr), "hipFree");
+}
+
+int32_t galois_hip_htod_sync_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    GH_REQUIRE_CTX(ctx);
+    if (bytes == 0) return GALOIS_HIP_OK;
+    GH_REQUIRE(ctx, dst_dev && src_host, GALOIS_HIP_E_NULL, "htod_sync_copy");
+    GH_BIND(ctx);
+    hipError_t e = hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipMemcpyAsync(H2D)");
+    return gh_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int32_t galois_hip_dtoh_sync_copy(galois_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    GH_REQUIRE_CTX(ctx);
+    if (bytes == 0) return GALOIS_HIP_OK;
+    GH_REQUIRE(ctx, dst_host && src_dev, GALOIS_HIP_E_NULL, "dtoh_sync_copy");
+    GH_BIND(ctx);
+    hipError_t e = hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipMemcpyAsync(D2H)");
+    return gh_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int32_t galois_hip_dtod_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
+    GH_REQUIRE_CTX(ctx);
+    if (bytes == 0) return GALOIS_HIP_OK;
+    GH_REQUIRE(ctx, dst_dev && src_dev, GALOIS_HIP_E_NULL, "dtod_copy");
+    GH_BIND(ctx);
+    return gh_hip(ctx, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream),
+                  "hipMemcpyAsync(D2D)");
+}
+
+int32_t galois_hip_dtod_copy_2d(galois_hip_ctx *ctx, void *dst_dev, size_t dpitch, const void *src_dev,
+                                size_t spitch, size_t width_bytes, size_t height) {
+    GH_REQUIRE_CTX(ctx);
+    if (width_bytes == 0 || height == 0) return GALOIS_HIP_OK;
+    GH_REQUIRE(ctx, dst_dev && src_dev, GALOIS_HIP_E_NULL, "dtod_copy_2d");
+    GH_REQUIRE(ctx, dpitch >= width_bytes && spitch >= width_bytes, GALOIS_HIP_E_SHAPE, "dtod_copy_2d: pitch < width");
+    GH_BIND(ctx);
+    return gh_hip(ctx,
+                  hipMemcpy2DAsync(dst_dev, dpitch, src_dev, spitch, width_bytes, height, hipMemcpyDeviceToDevice,
+                                   ctx->stream),
+                  "hipMemcpy2DAsync(D2D)");
+}
+
+int32_t galois_hip_synchronize(galois_hip_ctx *ctx) {
+    GH_REQUIRE_CTX(ctx);
+    GH_BIND(ctx);
+    return gh_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int32_t galois_hip_event_create(galois_hip_ctx *ctx, galois_hip_event **out) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, out != nullptr, GALOIS_HIP_E_NULL, "event_create: out");
+    GH_BIND(ctx);
+    galois_hip_event *ev = new galois_hip_event();
+    hipError_t e = hipEventCreate(&ev->ev);
+    if (e != hipSuccess) {
+        delete ev;
+        *out = nullptr;
+        return gh_hip(ctx, e, "hipEventCreate");
+    }
+    *out = ev;
+    return GALOIS_HIP_OK;
+}
+
+int32_t galois_hip_event_record(galois_hip_ctx *ctx, galois_hip_event *ev) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, ev != nullptr, GALOIS_HIP_E_NULL, "event_record");
+    GH_BIND(ctx);
+    return gh_hip(ctx, hipEventRecord(ev->ev, ctx->stream), "hipEventRecord");
+}
+
+int32_t galois_hip_event_elapsed_ms(galois_hip_ctx *ctx, galois_hip_event *start, galois_hip_event *stop, float *ms) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, start && stop && ms, GALOIS_HIP_E_NULL, "event_elapsed_ms");
+    GH_BIND(ctx);
+    hipError_t e = hipEventSynchronize(stop->ev);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipEventSynchronize");
+    return gh_hip(ctx, hipEventElapsedTime(ms, start->ev, stop->ev), "hipEventElapsedTime");
+}
+
+int32_t galois_hip_event_destroy(galois_hip_ctx *ctx, galois_hip_event *ev) {
+    GH_REQUIRE_CTX(ctx);
+    if (!ev) return GALOIS_HIP_OK;
+    GH_BIND(ctx);
+    hipError_t e = hipEventDestroy(ev->ev);
+    delete ev;
+    return gh_hip(ctx, e, "hipEventDestroy");
+}
+
+}  // extern "C"

@@ -1,0 +1,360 @@
+// Q4_0 x f32 matrix-vector product for decode: an HBM-bandwidth kernel for gfx950.
+//
+// Replaces dequantize_mul_mat_vec_q4_0 (galois-kernels/src/matmul.cu:45-117) and its
+// launcher (src/cuda.rs:1011-1034): dst[row] = sum_col (q-8)*d * y[col].
+//
+// Layout of the work.  Two consecutive 18-byte blocks form a 36-byte "slot" that is
+// 4-byte aligned whenever K % 64 == 0, so a lane fetches one slot of one row with
+// dwordx4 + dwordx4 + dword loads and the 64 lanes of a wave cover 2304 contiguous
+// bytes (4096 weights) of that row.  The weight nibbles are never unpacked: a dword of
+// eight nibbles, XORed with 0x88888888 (which turns q into the 4-bit two's complement
+// of q-8), goes straight into v_dot8_i32_i4 against a dword holding one signed 4-bit
+// digit of eight activations.  The activations are converted once per workgroup into
+// block-scaled fixed point, split into L such digit planes (gemv_xprep.h) and kept in
+// registers for every row the wave owns.  Per block the integer sum is exact; it is
+// converted to f32 once and multiplied by the block's power-of-two activation scale
+// and the f16 weight scale d.
+#include "common.h"
+#include "gemv_xprep.h"
+
+// Phase timestamps for tuning builds (-DGEMV_TIMING): one s_memtime per phase per wave.
+#ifdef GEMV_TIMING
+__device__ unsigned long long *g_gemv_tbuf;
+#define GH_TSTAMP(i)                                                                                   \
+    do {                                                                                               \
+        if ((threadIdx.x & 63) == 0)                                                                   \
+            g_gemv_tbuf[((size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + (i)] = \
+                __builtin_amdgcn_s_memtime();                                                          \
+    } while (0)
+#else
+#define GH_TSTAMP(i)
+#endif
+
+namespace {
+
+constexpr int kChunkSlots = 192;  // slots staged per pass over LDS (12288 activations)
+
+struct __attribute__((aligned(4))) q4_slot {
+    uint32_t w[9];  // [d0 | qs0[0..1]] [qs0 2..5] [6..9] [10..13] [qs0 14..15 | d1] [qs1 0..3] .. [qs1 12..15]
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 64 lanes of a wave; every lane ends with the total.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_mov<0xB1>(v);   // quad_perm(1,0,3,2)
+    v += dpp_mov<0x4E>(v);   // quad_perm(2,3,0,1)
+    v += dpp_mov<0x141>(v);  // row_half_mirror
+    v += dpp_mov<0x140>(v);  // row_mirror
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+
+__device__ __forceinline__ void load_slot(q4_slot &q, const uint8_t *p) {
+    const uint32_t *s = reinterpret_cast<const uint32_t *>(p);
+#pragma unroll
+    for (int i = 0; i < 9; i++) q.w[i] = s[i];  // plain loads: the three loads of a lane share cache lines
+}
+
+// LDS image of one prepared slot: L planes x 8 dwords, then the two block scales.
+template <int L>
+struct slot_lds {
+    static constexpr int dwords = 8 * L + 4;  // stride = 4 (mod 8): 16-byte reads of 8 lanes hit 32 distinct banks
+};
+
+// Sum over the 64 lanes of a wave with DPP only; the total lands in lane 63.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+    v += dpp_mov<0x111>(v);  // row_shr:1
+    v += dpp_mov<0x112>(v);  // row_shr:2
+    v += dpp_mov<0x114>(v);  // row_shr:4
+    v += dpp_mov<0x118>(v);  // row_shr:8  -> lane 15 of each row holds the row total
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));  // row_bcast:15
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));  // row_bcast:31
+    return v;
+}
+
+// Activation preparation, split in two so that the activation loads can be issued before
+// the first weight loads (loads return in order, so whatever must be consumed first has to
+// be requested first) and the arithmetic runs while the weights are in flight.
+// One thread per (slot, weight-dword group); a quad of threads covers one block.
+template <int L, int THREADS, int PG>  // PG: groups per thread, an upper bound fixed at dispatch
+struct xprep_state {
+    float2 v[PG][4];
+
+    __device__ __forceinline__ void load(const float *__restrict__ xg, int c0, int cs) {
+#pragma unroll
+        for (int p = 0; p < PG; p++) {
+            const int idx = threadIdx.x + p * THREADS;
+            if (idx < cs * 8) {
+                const int slot = idx >> 3, g = idx & 7;
+                const float *xs = xg + (size_t)(c0 + slot) * 64;
+#pragma unroll
+                for (int t = 0; t < 4; t += 2) {
+                    // nibble pairs t, t+1 of group g: weights (b, b+1) low nibbles and (16+b, 17+b) high nibbles
+                    const int b = xprep::group_x_index(g, 2 * t);  // even by construction
+                    v[p][t] = *reinterpret_cast<const float2 *>(xs + b);
+                    v[p][t + 1] = *reinterpret_cast<const float2 *>(xs + b + 16);
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void compute(uint32_t *lds, int cs) const {
+#pragma unroll
+        for (int p = 0; p < PG; p++) {
+            const int idx = threadIdx.x + p * THREADS;
+            if (idx < cs * 8) {
+                const int slot = idx >> 3, g = idx & 7;
+                // nibble order of the weight dword: byte b low, byte b high, byte b+1 low, byte b+1 high, ...
+                const float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
+                                     v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
+                // max of |x| on the bit patterns: for non-negative floats the unsigned order is the numeric
+                // order, with inf and NaN on top, so a non-finite activation is never lost
+                uint32_t amax = 0;
+#pragma unroll
+                for (int j = 0; j < 8; j++) amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
+                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0xB1, 0xF, 0xF, true));
+                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0x4E, 0xF, 0xF, true));
+                float mult, scale;
+                xprep::block_scales<L>(amax, &mult, &scale);
+                uint32_t planes[L];
+                xprep::make_planes<L>(x8, mult, planes);
+                uint32_t *dst = lds + slot * slot_lds<L>::dwords;
+#pragma unroll
+                for (int l = 0; l < L; l++) dst[l * 8 + g] = planes[l];
+                if ((g & 3) == 0) dst[8 * L + (g >> 2)] = __builtin_bit_cast(uint32_t, scale);
+            }
+        }
+    }
+};
+
+__device__ __forceinline__ int sdot8_first(uint32_t a, uint32_t b) {
+    int d;
+    asm("v_dot8_i32_i4 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+
+// Integer dot of one block's four nibble dwords with its L planes: sum_l 16^l * dot8.
+// One accumulator per plane, issued round-robin: back-to-back v_dot8 into the same
+// register serialise on the dot pipeline's latency, independent ones issue every cycle.
+template <int L>
+__device__ __forceinline__ int block_dot(const uint32_t nd[4], const uint32_t (&xl)[L][8], int base) {
+    int t[L];
+#pragma unroll
+    for (int l = 0; l < L; l++) t[l] = sdot8_first(nd[0], xl[l][base]);
+#pragma unroll
+    for (int i = 1; i < 4; i++)
+#pragma unroll
+        for (int l = 0; l < L; l++) t[l] = __builtin_amdgcn_sdot8((int)nd[i], (int)xl[l][base + i], t[l], false);
+    int r = t[L - 1];
+#pragma unroll
+    for (int l = L - 2; l >= 0; l--) r = (r << 4) + t[l];
+    return r;
+}
+
+template <int L>
+__device__ __forceinline__ float slot_dot(const q4_slot &q, const uint32_t (&xl)[L][8], float sA, float sB) {
+    const float dA = f16_bits_to_f32(q.w[0] & 0xFFFFu);
+    const float dB = f16_bits_to_f32(q.w[4] >> 16);
+    const uint32_t sign = 0x88888888u;
+    // block A: qs bytes 0,1 sit in the top half of w[0], bytes 14,15 in the low half of w[4]
+    const uint32_t ndA[4] = {__builtin_amdgcn_alignbit(q.w[4], q.w[0], 16) ^ sign, q.w[1] ^ sign, q.w[2] ^ sign,
+                             q.w[3] ^ sign};
+    const uint32_t ndB[4] = {q.w[5] ^ sign, q.w[6] ^ sign, q.w[7] ^ sign, q.w[8] ^ sign};
+    const int tA = block_dot<L>(ndA, xl, 0);
+    const int tB = block_dot<L>(ndB, xl, 4);
+    float r = (dA * sA) * (float)tA;
+    r = __builtin_fmaf(dB * sB, (float)tB, r);
+    return r;
+}
+
+// Fast path: K % 64 == 0, W 4-byte aligned, x 8-byte aligned.
+// Each wave owns R*G consecutive rows; a workgroup owns WAVES*R*G rows.  No explicit
+// register double-buffering: several workgroups share a CU and overlap each other's
+// loads, activation preparation and arithmetic.
+// PG bounds the activation groups one thread prepares per pass; OCC is the number of waves
+// per SIMD the register allocation must leave room for.
+// MULTIPASS: K exceeds one LDS pass (kChunkSlots slots); the single-pass instantiation has
+// no outer loop, which keeps the compiler from ordering loads across a back edge.
+template <int L, int R, int G, int WAVES, int PG, int OCC, bool MULTIPASS>
+__global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t *__restrict__ W,
+                                                             const float *__restrict__ xg, float *__restrict__ y,
+                                                             int nslots, int N) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    constexpr int SD = slot_lds<L>::dwords;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int row0 = (blockIdx.x * WAVES + wave) * (R * G);
+    const size_t row_bytes = (size_t)nslots * sizeof(q4_slot);
+
+    float acc[G][R];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[g][r] = 0.0f;
+    GH_TSTAMP(0);
+
+    for (int c0 = 0; c0 < (MULTIPASS ? nslots : 1); c0 += kChunkSlots) {
+        const int cs = MULTIPASS ? min(kChunkSlots, nslots - c0) : nslots;
+        if (MULTIPASS && c0 > 0) __syncthreads();
+        xprep_state<L, WAVES * 64, PG> xp;
+        xp.load(xg, c0, cs);
+        // first weights of this pass go in flight behind the activations
+        q4_slot q0[R];
+        {
+            const int s = min(c0 + lane, nslots - 1);
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                load_slot(q0[r], W + (size_t)min(row0 + r, N - 1) * row_bytes + (size_t)s * sizeof(q4_slot));
+        }
+        GH_TSTAMP(1);
+        xp.compute(lds, cs);
+        GH_TSTAMP(2);
+        __syncthreads();
+        GH_TSTAMP(3);
+
+        for (int sl = lane; sl - lane < cs; sl += 64) {  // uniform trip count; lanes past the end idle
+            const bool act = sl < cs;
+            const int s_ld = min(sl, cs - 1);
+            uint32_t xl[L][8];
+            float sA, sB;
+            {
+                const uint32_t *src = lds + s_ld * SD;
+#pragma unroll
+                for (int l = 0; l < L; l++) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(src + l * 8);
+                    const uint4 b = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
+                    xl[l][0] = a.x, xl[l][1] = a.y, xl[l][2] = a.z, xl[l][3] = a.w;
+                    xl[l][4] = b.x, xl[l][5] = b.y, xl[l][6] = b.z, xl[l][7] = b.w;
+                }
+                const uint2 sc = *reinterpret_cast<const uint2 *>(src + 8 * L);
+                sA = __builtin_bit_cast(float, sc.x);
+                sB = __builtin_bit_cast(float, sc.y);
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                q4_slot q[R];
+                if (g == 0 && sl == lane) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) q[r] = q0[r];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < R; r++)  // rows past N are loaded from row N-1 and never stored
+                        load_slot(q[r], W + (size_t)min(row0 + g * R + r, N - 1) * row_bytes +
+                                            (size_t)(c0 + s_ld) * sizeof(q4_slot));
+                }
+                if (act) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) acc[g][r] += slot_dot<L>(q[r], xl, sA, sB);
+                }
+            }
+        }
+    }
+
+    GH_TSTAMP(4);
+    // every total lands in lane 63; lane 63-j picks up row j so the wave stores its rows at once
+    float out = 0.0f;
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float t = wave_sum_to_lane63(acc[g][r]);
+            const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
+            if (lane == g * R + r) out = b;
+        }
+    if (lane < R * G && row0 + lane < N) y[row0 + lane] = out;
+    GH_TSTAMP(5);
+}
+
+// Generic path: any K % 32 == 0 and any 2-byte-aligned W / 4-byte-aligned x.
+// One wave per row, one block per lane per step, 2-byte loads, plain f32 arithmetic.
+__global__ __launch_bounds__(256) void gemv_q4_0_generic(const uint16_t *__restrict__ W, const float *__restrict__ x,
+                                                        float *__restrict__ y, int nblocks, int N) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const uint16_t *wr = W + (size_t)row * nblocks * 9;
+    float acc = 0.0f;
+    for (int b = lane; b < nblocks; b += 64) {
+        const uint16_t *p = wr + (size_t)b * 9;
+        const float d = f16_bits_to_f32(p[0]);
+        const float *xb = x + (size_t)b * 32;
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t v = p[1 + j];  // bytes 2j, 2j+1
+            s = __builtin_fmaf((float)((int)(v & 0xF) - 8), xb[2 * j], s);
+            s = __builtin_fmaf((float)((int)((v >> 4) & 0xF) - 8), xb[2 * j + 16], s);
+            s = __builtin_fmaf((float)((int)((v >> 8) & 0xF) - 8), xb[2 * j + 1], s);
+            s = __builtin_fmaf((float)((int)((v >> 12) & 0xF) - 8), xb[2 * j + 17], s);
+        }
+        acc = __builtin_fmaf(d, s, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) y[row] = acc;
+}
+
+template <int L, int R, int G, int WAVES, int OCC>
+void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst, int nslots, int N) {
+    const int rows_per_wg = WAVES * R * G;
+    const dim3 grid((N + rows_per_wg - 1) / rows_per_wg), block(WAVES * 64);
+    const int pass_slots = min(nslots, kChunkSlots);
+    const size_t lds = (size_t)pass_slots * slot_lds<L>::dwords * sizeof(uint32_t);
+    constexpr int PGMAX = (kChunkSlots * 8 + WAVES * 64 - 1) / (WAVES * 64);
+    constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
+    const uint8_t *W = (const uint8_t *)vx;
+    if (nslots <= 64)
+        hipLaunchKernelGGL((gemv_q4_0_dot8<L, R, G, WAVES, PGSMALL, OCC, false>), grid, block, lds, ctx->stream, W,
+                           x, dst, nslots, N);
+    else if (nslots <= kChunkSlots)
+        hipLaunchKernelGGL((gemv_q4_0_dot8<L, R, G, WAVES, PGMAX, OCC, false>), grid, block, lds, ctx->stream, W, x,
+                           dst, nslots, N);
+    else
+        hipLaunchKernelGGL((gemv_q4_0_dot8<L, R, G, WAVES, PGMAX, OCC, true>), grid, block, lds, ctx->stream, W, x,
+                           dst, nslots, N);
+}
+
+}  // namespace
+
+extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, const void *vx, const float *y,
+                                                          float *dst, int32_t ncols, int32_t nrows) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, vx && y && dst, GALOIS_HIP_E_NULL, "dequantize_mul_mat_vec_q4_0");
+    GH_REQUIRE(ctx, ncols > 0 && nrows > 0 && ncols % 32 == 0, GALOIS_HIP_E_SHAPE,
+               "dequantize_mul_mat_vec_q4_0: ncols must be a positive multiple of 32, nrows positive");
+    GH_REQUIRE(ctx, gh_aligned(vx, 2) && gh_aligned(y, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN,
+               "dequantize_mul_mat_vec_q4_0");
+    GH_BIND(ctx);
+    const bool fast = (ncols % 64 == 0) && gh_aligned(vx, 4) && gh_aligned(y, 8);
+    if (fast) {
+        const int nslots = ncols / 64;
+        // Workgroup shape by rows per CU: few rows -> 16 waves x 1 row so every SIMD has work and the
+        // activation preparation is spread over 1024 threads; more rows -> 8 waves x 2 rows, several
+        // workgroups resident per CU so one's preparation overlaps another's streaming.
+        int cfg = ctx->gemv_config;
+        if (cfg == 0) {
+            const int64_t rows_per_cu = ((int64_t)nrows + ctx->n_cu - 1) / ctx->n_cu;
+            cfg = rows_per_cu <= 16 ? 1 : 4;
+        }
+        switch (cfg) {
+            case 1: launch_dot8<5, 1, 1, 16, 4>(ctx, vx, y, dst, nslots, nrows); break;  // 16 rows per workgroup
+            case 2: launch_dot8<5, 4, 1, 4, 2>(ctx, vx, y, dst, nslots, nrows); break;   // 16 rows, 4 waves
+            case 3: launch_dot8<5, 4, 1, 8, 3>(ctx, vx, y, dst, nslots, nrows); break;   // 32 rows per workgroup
+            case 4: launch_dot8<5, 2, 1, 8, 4>(ctx, vx, y, dst, nslots, nrows); break;   // 16 rows, 8 waves
+            case 5: launch_dot8<6, 4, 1, 4, 2>(ctx, vx, y, dst, nslots, nrows); break;   // 6 activation limbs
+            default: return gh_fail(ctx, GALOIS_HIP_E_UNSUPPORTED, "GALOIS_HIP_GEMV_CONFIG value");
+        }
+    } else {
+        hipLaunchKernelGGL(gemv_q4_0_generic, dim3((nrows + 3) / 4), dim3(256), 0, ctx->stream, (const uint16_t *)vx,
+                           y, dst, ncols / 32, nrows);
+    }
+    GH_LAUNCH_CHECK(ctx, "dequantize_mul_mat_vec_q4_0 launch");
+}

@@ -1,0 +1,115 @@
+// Activation preparation for the Q4_0 decode GEMV: f32 -> signed 4-bit limb planes.
+//
+// The GEMV multiplies 4-bit weights with v_dot8_i32_i4 (eight int4 x int4 products per
+// lane per instruction).  For that the f32 activations of one Q4_0 block (32 values) are
+// turned into a block-scaled fixed-point integer X = rne(x * 2^(XBITS-1-e)), where
+// 2^e <= max|x| < 2^(e+1), and X is written in balanced base 16: X = sum_l s_l * 16^l
+// with every digit s_l in [-8, 7].  Digit l of eight activations is packed into one dword
+// ("limb plane") in the nibble order of the weight dword they multiply, so that
+//     sum_k (q_k - 8) * x_k  =  2^(e-XBITS+1) * sum_l 16^l * dot8(weights ^ 0x88888888, plane_l)
+// holds exactly in integer arithmetic; the only rounding is that of x to XBITS-1 fractional
+// bits below its block's leading power of two (2^-21 relative for 6 limbs).
+//
+// Plain C++ (no HIP builtins) so the same code is unit-tested on the CPU.
+#pragma once
+#include <stdint.h>
+#include <string.h>
+
+#ifdef __HIPCC__
+#define GH_HD __host__ __device__ __forceinline__
+#else
+#define GH_HD inline
+#endif
+
+namespace xprep {
+
+template <int L>
+struct limb_cfg {
+    static_assert(L >= 2 && L <= 6, "2..6 limbs");
+    static constexpr int xbits = 4 * L - 2;                                  // |X| <= 2^xbits
+    static constexpr uint32_t bias = (uint32_t)(0x88888888ull >> (4 * (8 - L)));  // 8 in each of L digits
+};
+
+GH_HD uint32_t f32_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+GH_HD float bits_f32(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+// Byte of the 16-byte qs array that nibble pair t (0..3) of weight-dword group g (0..7) holds.
+// A 36-byte slot is two blocks: block A's qs start 2 bytes into the slot, so its bytes
+// 0,1 and 14,15 share dwords with the two f16 scales and are gathered into group 0
+// ("edge"); groups 1..3 are bytes 2-5, 6-9, 10-13; block B's groups 4..7 are aligned.
+GH_HD int group_byte(int g, int t) {
+    if (g >= 4) return 4 * (g - 4) + t;
+    if (g == 0) return t < 2 ? t : 12 + t;
+    return 4 * g - 2 + t;
+}
+
+// Index (within the 64 activations of a slot) of nibble j (0..7) of group g:
+// even nibbles are the low nibbles (weight b), odd nibbles the high nibbles (weight 16+b).
+GH_HD int group_x_index(int g, int j) { return (g >= 4 ? 32 : 0) + group_byte(g, j >> 1) + ((j & 1) ? 16 : 0); }
+
+// Scale pair for a block whose max|x| has f32 bits `amax_bits`: `mult` maps x to the integer
+// grid, `scale` maps integer dot products back.  Both are powers of two (or 0 / NaN).
+template <int L>
+GH_HD void block_scales(uint32_t amax_bits, float *mult, float *scale) {
+    const int eb = (int)((amax_bits >> 23) & 0xFF);
+    constexpr int xb = limb_cfg<L>::xbits;
+    if (eb == 255) {  // inf or nan in the block: poison the block's contribution
+        *mult = 0.0f;
+        *scale = bits_f32(0x7FC00000u);
+    } else if (eb <= xb) {  // zero, subnormal or below 2^-100: contributes nothing representable
+        *mult = 0.0f;
+        *scale = 0.0f;
+    } else {
+        *mult = bits_f32((uint32_t)(253 + xb - eb) << 23);
+        *scale = bits_f32((uint32_t)(eb - xb + 1) << 23);
+    }
+}
+
+// x * mult rounded to nearest-even integer, offset by `bias`, digits made signed:
+// returns the L balanced digits of X as packed 4-bit two's-complement nibbles.
+template <int L>
+GH_HD uint32_t signed_digits(float x, float mult) {
+    const float f = __builtin_fmaf(x, mult, 12582912.0f);  // 1.5 * 2^23: integer lands in the mantissa
+    const uint32_t y = f32_bits(f) - 0x4B400000u + limb_cfg<L>::bias;
+    return y ^ limb_cfg<L>::bias;
+}
+
+// 8x8 nibble transpose: in[j] nibble l  ->  out[l] nibble j.
+GH_HD void transpose_nibbles(const uint32_t in[8], uint32_t out[8]) {
+    uint32_t a[8], b[8];
+    // 4x4 blocks of nibbles (16-bit halves) between rows j and j+4
+    for (int j = 0; j < 4; j++) {
+        a[j] = (in[j] & 0x0000FFFFu) | (in[j + 4] << 16);
+        a[j + 4] = (in[j] >> 16) | (in[j + 4] & 0xFFFF0000u);
+    }
+    // 2x2 blocks (bytes) between rows j and j+2
+    for (int h = 0; h < 8; h += 4)
+        for (int j = h; j < h + 2; j++) {
+            b[j] = (a[j] & 0x00FF00FFu) | ((a[j + 2] & 0x00FF00FFu) << 8);
+            b[j + 2] = ((a[j] >> 8) & 0x00FF00FFu) | (a[j + 2] & 0xFF00FF00u);
+        }
+    // single nibbles between rows j and j+1
+    for (int j = 0; j < 8; j += 2) {
+        out[j] = (b[j] & 0x0F0F0F0Fu) | ((b[j + 1] & 0x0F0F0F0Fu) << 4);
+        out[j + 1] = ((b[j] >> 4) & 0x0F0F0F0Fu) | (b[j + 1] & 0xF0F0F0F0u);
+    }
+}
+
+// Eight activations (already in nibble order of their weight dword) -> L limb planes.
+template <int L>
+GH_HD void make_planes(const float x[8], float mult, uint32_t planes[L]) {
+    uint32_t s[8], t[8];
+    for (int j = 0; j < 8; j++) s[j] = signed_digits<L>(x[j], mult);
+    transpose_nibbles(s, t);
+    for (int l = 0; l < L; l++) planes[l] = t[l];
+}
+
+}  // namespace xprep

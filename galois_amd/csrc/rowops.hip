@@ -1,0 +1,313 @@
+// Single-pass row kernels for gfx950: RMSNorm (+ fused weight), RoPE, softmax (+ causal).
+// Each reads its input once from HBM and writes its output once; rows live in registers.
+#include "common.h"
+
+namespace {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_mov<0xB1>(v);   // quad_perm(1,0,3,2)
+    v += dpp_mov<0x4E>(v);   // quad_perm(2,3,0,1)
+    v += dpp_mov<0x141>(v);  // row_half_mirror
+    v += dpp_mov<0x140>(v);  // row_mirror
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_mov<0xB1>(v));
+    v = fmaxf(v, dpp_mov<0x4E>(v));
+    v = fmaxf(v, dpp_mov<0x141>(v));
+    v = fmaxf(v, dpp_mov<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// rms_norm_f32 (galois-kernels/src/rms_norm.cu:13-49) with the optional broadcast
+// weight of mul_f32 (mul.cu:3-12) fused in.  One workgroup per row; the row is
+// read once into registers (NV float4 per thread), reduced, scaled and written.
+constexpr int kNormThreads = 256;
+
+template <int NV>
+__global__ __launch_bounds__(kNormThreads) void rms_norm_rows(const float *__restrict__ x,
+                                                              const float *__restrict__ w,
+                                                              float *__restrict__ y, int ncols, float eps) {
+    __shared__ float part[kNormThreads / 64];
+    const size_t base = (size_t)blockIdx.x * ncols;
+    const int nvec = ncols >> 2;
+    float4 v[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = threadIdx.x + i * kNormThreads;
+        v[i] = c < nvec ? reinterpret_cast<const float4 *>(x + base)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kNormThreads / 64; i++) tot += part[i];
+    const float scale = 1.0f / sqrtf(tot / (float)ncols + eps);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = threadIdx.x + i * kNormThreads;
+        if (c < nvec) {
+            float4 o = make_float4(v[i].x * scale, v[i].y * scale, v[i].z * scale, v[i].w * scale);
+            if (w) {
+                const float4 g = reinterpret_cast<const float4 *>(w)[c];
+                o.x *= g.x, o.y *= g.y, o.z *= g.z, o.w *= g.w;
+            }
+            reinterpret_cast<float4 *>(y + base)[c] = o;
+        }
+    }
+}
+
+// Any ncols / alignment: the row is read twice (the second read hits L2).
+__global__ __launch_bounds__(kNormThreads) void rms_norm_rows_generic(const float *__restrict__ x,
+                                                                      const float *__restrict__ w,
+                                                                      float *__restrict__ y, int ncols, float eps) {
+    __shared__ float part[kNormThreads / 64];
+    const size_t base = (size_t)blockIdx.x * ncols;
+    float ss = 0.0f;
+    for (int c = threadIdx.x; c < ncols; c += kNormThreads) ss += x[base + c] * x[base + c];
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kNormThreads / 64; i++) tot += part[i];
+    const float scale = 1.0f / sqrtf(tot / (float)ncols + eps);
+    for (int c = threadIdx.x; c < ncols; c += kNormThreads) {
+        float o = x[base + c] * scale;
+        if (w) o *= w[c];
+        y[base + c] = o;
+    }
+}
+
+int32_t launch_rms_norm(galois_hip_ctx *ctx, const float *x, const float *w, float *dst, int32_t ncols,
+                        int32_t nrows, float eps, const char *what) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && dst, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, ncols > 0 && nrows > 0, GALOIS_HIP_E_SHAPE, what);
+    GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(dst, 4) && gh_aligned(w, 4), GALOIS_HIP_E_ALIGN, what);
+    GH_BIND(ctx);
+    const bool vec = ncols % 4 == 0 && gh_aligned(x, 16) && gh_aligned(dst, 16) && gh_aligned(w, 16);
+    const int nv = (ncols / 4 + kNormThreads - 1) / kNormThreads;
+    const dim3 grid(nrows), block(kNormThreads);
+    if (vec && nv <= 1)
+        hipLaunchKernelGGL(rms_norm_rows<1>, grid, block, 0, ctx->stream, x, w, dst, ncols, eps);
+    else if (vec && nv <= 2)
+        hipLaunchKernelGGL(rms_norm_rows<2>, grid, block, 0, ctx->stream, x, w, dst, ncols, eps);
+    else if (vec && nv <= 4)
+        hipLaunchKernelGGL(rms_norm_rows<4>, grid, block, 0, ctx->stream, x, w, dst, ncols, eps);
+    else if (vec && nv <= 8)
+        hipLaunchKernelGGL(rms_norm_rows<8>, grid, block, 0, ctx->stream, x, w, dst, ncols, eps);
+    else if (vec && nv <= 16)
+        hipLaunchKernelGGL(rms_norm_rows<16>, grid, block, 0, ctx->stream, x, w, dst, ncols, eps);
+    else
+        hipLaunchKernelGGL(rms_norm_rows_generic, grid, block, 0, ctx->stream, x, w, dst, ncols, eps);
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
+// ------------------------------------------------------------------ RoPE
+// rope_f32 (galois-kernels/src/rope.cu:3-28): adjacent pairs, one position per group of
+// p_delta_rows consecutive rows.  One workgroup per position group; a lane computes
+// sin/cos for its pair index once and reuses it for every row (head) of the group, so
+// the transcendental cost is shared by all heads.  theta follows the reference formula
+// in f32: pos * freq_scale * powf(theta_scale, pair).
+constexpr int kRopeThreads = 256;
+
+__global__ __launch_bounds__(kRopeThreads) void rope_rows(const float *__restrict__ x, float *__restrict__ y,
+                                                          int ncols, int nrows, const int32_t *__restrict__ pos,
+                                                          float freq_scale, int p_delta_rows, float theta_scale) {
+    const int group = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int npairs = ncols >> 1;
+    const int row_lo = group * p_delta_rows;
+    const int row_hi = min(row_lo + p_delta_rows, nrows);
+    const float p0 = (float)pos[group] * freq_scale;
+    for (int pi = lane; pi < npairs; pi += 64) {
+        const float theta = p0 * powf(theta_scale, (float)pi);
+        float sn, cs;
+        sincosf(theta, &sn, &cs);
+        int r = row_lo + wave;
+        // four rows in flight per lane
+        for (; r + 3 * (kRopeThreads / 64) < row_hi; r += 4 * (kRopeThreads / 64)) {
+            float2 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                v[u] = reinterpret_cast<const float2 *>(x + (size_t)(r + u * (kRopeThreads / 64)) * ncols)[pi];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                reinterpret_cast<float2 *>(y + (size_t)(r + u * (kRopeThreads / 64)) * ncols)[pi] =
+                    make_float2(v[u].x * cs - v[u].y * sn, v[u].x * sn + v[u].y * cs);
+        }
+        for (; r < row_hi; r += kRopeThreads / 64) {
+            const float2 v = reinterpret_cast<const float2 *>(x + (size_t)r * ncols)[pi];
+            reinterpret_cast<float2 *>(y + (size_t)r * ncols)[pi] =
+                make_float2(v.x * cs - v.y * sn, v.x * sn + v.y * cs);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ softmax
+// soft_max_f32 (galois-kernels/src/softmax.cu:3-48): f32 row softmax, -inf inputs are
+// masked.  One wave per row, the row held in registers (NV float4 per lane): one read,
+// one write.  `causal` computes the mask from indices instead: row r keeps columns
+// <= n_past + (r % rows_per_head); masked inputs are not read and their outputs are 0.
+constexpr int kSoftThreads = 256;
+
+template <int NV>
+__global__ __launch_bounds__(kSoftThreads) void soft_max_rows(const float *__restrict__ x, float *__restrict__ y,
+                                                              int ncols, int nrows, int causal, int rows_per_head,
+                                                              int n_past) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * (kSoftThreads / 64) + (threadIdx.x >> 6);
+    if (row >= nrows) return;
+    const int nvalid = causal ? min(ncols, n_past + (row % rows_per_head) + 1) : ncols;
+    const size_t base = (size_t)row * ncols;
+    const float ninf = -__builtin_inff();
+    float4 v[NV];
+    float mx = ninf;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = (lane + i * 64) * 4;
+        if (c < nvalid) {
+            v[i] = *reinterpret_cast<const float4 *>(x + base + c);
+            if (c + 1 >= nvalid) v[i].y = ninf;
+            if (c + 2 >= nvalid) v[i].z = ninf;
+            if (c + 3 >= nvalid) v[i].w = ninf;
+        } else {
+            v[i] = make_float4(ninf, ninf, ninf, ninf);
+        }
+        mx = fmaxf(mx, fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)));
+    }
+    mx = wave_max(mx);
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        v[i].x = expf(v[i].x - mx);
+        v[i].y = expf(v[i].y - mx);
+        v[i].z = expf(v[i].z - mx);
+        v[i].w = expf(v[i].w - mx);
+        sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = (lane + i * 64) * 4;
+        if (c < ncols)
+            *reinterpret_cast<float4 *>(y + base + c) =
+                make_float4(v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+    }
+}
+
+// Any ncols / alignment: one workgroup per row, three passes (re-reads hit L2).
+__global__ __launch_bounds__(kSoftThreads) void soft_max_rows_generic(const float *__restrict__ x,
+                                                                      float *__restrict__ y, int ncols, int causal,
+                                                                      int rows_per_head, int n_past) {
+    __shared__ float part[kSoftThreads / 64];
+    const int row = blockIdx.x;
+    const int nvalid = causal ? min(ncols, n_past + (row % rows_per_head) + 1) : ncols;
+    const size_t base = (size_t)row * ncols;
+    float mx = -__builtin_inff();
+    for (int c = threadIdx.x; c < nvalid; c += kSoftThreads) mx = fmaxf(mx, x[base + c]);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = part[0];
+#pragma unroll
+    for (int i = 1; i < kSoftThreads / 64; i++) mx = fmaxf(mx, part[i]);
+    __syncthreads();
+    float sum = 0.0f;
+    for (int c = threadIdx.x; c < nvalid; c += kSoftThreads) sum += expf(x[base + c] - mx);
+    sum = wave_sum(sum);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kSoftThreads / 64; i++) tot += part[i];
+    const float inv = 1.0f / tot;
+    for (int c = threadIdx.x; c < ncols; c += kSoftThreads)
+        y[base + c] = c < nvalid ? expf(x[base + c] - mx) * inv : 0.0f;
+}
+
+int32_t launch_soft_max(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols, int32_t nrows, int causal,
+                        int32_t rows_per_head, int32_t n_past, const char *what) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && dst, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, ncols > 0 && nrows > 0, GALOIS_HIP_E_SHAPE, what);
+    GH_REQUIRE(ctx, !causal || (rows_per_head > 0 && n_past >= 0), GALOIS_HIP_E_SHAPE, what);
+    GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, what);
+    GH_BIND(ctx);
+    const bool vec = ncols % 4 == 0 && gh_aligned(x, 16) && gh_aligned(dst, 16);
+    const int nv = (ncols / 4 + 63) / 64;
+    const dim3 grid((nrows + kSoftThreads / 64 - 1) / (kSoftThreads / 64)), block(kSoftThreads);
+#define GH_SOFT(NV) \
+    hipLaunchKernelGGL(soft_max_rows<NV>, grid, block, 0, ctx->stream, x, dst, ncols, nrows, causal, rows_per_head, n_past)
+    if (vec && nv <= 1)
+        GH_SOFT(1);
+    else if (vec && nv <= 2)
+        GH_SOFT(2);
+    else if (vec && nv <= 4)
+        GH_SOFT(4);
+    else if (vec && nv <= 8)
+        GH_SOFT(8);
+    else if (vec && nv <= 16)
+        GH_SOFT(16);
+    else
+        hipLaunchKernelGGL(soft_max_rows_generic, dim3(nrows), block, 0, ctx->stream, x, dst, ncols, causal,
+                           rows_per_head, n_past);
+#undef GH_SOFT
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t galois_hip_rms_norm_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols, int32_t nrows,
+                                float eps) {
+    return launch_rms_norm(ctx, x, nullptr, dst, ncols, nrows, eps, "rms_norm_f32");
+}
+
+int32_t galois_hip_rms_norm_mul_f32(galois_hip_ctx *ctx, const float *x, const float *weight, float *dst,
+                                    int32_t ncols, int32_t nrows, float eps) {
+    if (ctx && !weight) return gh_fail(ctx, GALOIS_HIP_E_NULL, "rms_norm_mul_f32: weight");
+    return launch_rms_norm(ctx, x, weight, dst, ncols, nrows, eps, "rms_norm_mul_f32");
+}
+
+int32_t galois_hip_rope_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols, int32_t nrows,
+                            const int32_t *pos, float freq_scale, int32_t p_delta_rows, float theta_scale) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && dst && pos, GALOIS_HIP_E_NULL, "rope_f32");
+    GH_REQUIRE(ctx, ncols > 0 && ncols % 2 == 0 && nrows > 0 && p_delta_rows > 0, GALOIS_HIP_E_SHAPE,
+               "rope_f32: ncols must be even and positive, nrows and p_delta_rows positive");
+    GH_REQUIRE(ctx, gh_aligned(x, 8) && gh_aligned(dst, 8) && gh_aligned(pos, 4), GALOIS_HIP_E_ALIGN, "rope_f32");
+    GH_BIND(ctx);
+    const int groups = (nrows + p_delta_rows - 1) / p_delta_rows;
+    hipLaunchKernelGGL(rope_rows, dim3(groups), dim3(kRopeThreads), 0, ctx->stream, x, dst, ncols, nrows, pos,
+                       freq_scale, p_delta_rows, theta_scale);
+    GH_LAUNCH_CHECK(ctx, "rope_f32 launch");
+}
+
+int32_t galois_hip_soft_max_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols, int32_t nrows) {
+    return launch_soft_max(ctx, x, dst, ncols, nrows, 0, 1, 0, "soft_max_f32");
+}
+
+int32_t galois_hip_soft_max_causal_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols,
+                                       int32_t rows_per_head, int32_t nrows, int32_t n_past) {
+    return launch_soft_max(ctx, x, dst, ncols, nrows, 1, rows_per_head, n_past, "soft_max_causal_f32");
+}
+
+}  // extern "C"

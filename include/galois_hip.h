@@ -1,0 +1,137 @@
+/*
+ * galois_hip.h -- C ABI of the MI355X (gfx950) backend for galois's Q4_0 path.
+ *
+ * This is what a rewritten src/cuda.rs binds with `extern "C"` in place of
+ * cudarc + galois_kernels + cuBLAS.  Plain pointers and sizes only.  Every
+ * entry point cites the reference interface it replaces (paths relative to the
+ * szuwgh/galois tree).
+ *
+ * Conventions
+ *   - Every function returns a status: 0 = ok, negative = GALOIS_HIP_E_* (argument
+ *     errors detected on the host before anything is launched), positive = the
+ *     hipError_t that HIP reported.  Nothing aborts or throws across the boundary
+ *     (the reference panics via todo!()/unwrap(), src/cuda.rs:305,611,805).
+ *   - A context owns one device ordinal and one HIP stream (the reference uses
+ *     cudarc's single default stream, src/cuda.rs:221-229).  All op entry points
+ *     are asynchronous on that stream; only *_sync_copy and synchronize block.
+ *     A context is thread-compatible: callers serialise access, as the
+ *     reference's &mut dst borrow rules do.
+ *   - Tensors are raw device pointers.  Q4_0 data keeps the reference's block
+ *     bytes exactly (src/ggml_quants.rs:140-145, galois-kernels/src/matmul.cu:19-23):
+ *     18 bytes per 32 weights = f16 scale d, then qs[16]; weight j is the low
+ *     nibble of qs[j], weight j+16 the high nibble; value = (nibble - 8) * d.
+ *   - Shapes are explicit int32/int64 (the reference passes usize where its
+ *     kernels declare int, src/cuda.rs:1032 vs matmul.cu:45).
+ */
+#ifndef GALOIS_HIP_H
+#define GALOIS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GALOIS_HIP_ABI_VERSION 1
+
+#define GALOIS_HIP_OK 0
+#define GALOIS_HIP_E_NULL (-1)      /* a required pointer is NULL */
+#define GALOIS_HIP_E_SHAPE (-2)     /* a dimension is <= 0, too large, or not a multiple the op needs */
+#define GALOIS_HIP_E_ALIGN (-3)     /* a device pointer is not aligned as the op needs */
+#define GALOIS_HIP_E_ORDINAL (-4)   /* no such device */
+#define GALOIS_HIP_E_UNSUPPORTED (-5) /* the reference leaves this combination todo!() and so do we */
+#define GALOIS_HIP_E_ARCH (-6)      /* the device is not gfx950 */
+
+typedef struct galois_hip_ctx galois_hip_ctx;
+typedef struct galois_hip_event galois_hip_event;
+
+/* ---- device / stream / buffer layer -------------------------------------- */
+
+/* CudaDevice::new(ordinal), src/cuda.rs:221-229: bind a device, create its stream. */
+int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out);
+int32_t galois_hip_destroy(galois_hip_ctx *ctx);
+/* init_cuda_function(&dev), src/kernels.rs:4-22.  Code objects are linked into
+ * the library, so nothing is loaded; this checks the ABI version and that the
+ * device can run them, and returns the number of kernels in *n_kernels. */
+int32_t galois_hip_init_functions(galois_hip_ctx *ctx, int32_t abi_version, int32_t *n_kernels);
+/* Text of the last non-zero status on this context ("" if none); never NULL. */
+const char *galois_hip_last_error(const galois_hip_ctx *ctx);
+/* Name for a status code of this ABI (valid without a context). */
+const char *galois_hip_status_string(int32_t status);
+/* Device properties the harness prints: name/arch string, CU count, clocks (kHz), memory bytes. */
+int32_t galois_hip_device_info(galois_hip_ctx *ctx, char *name, int32_t name_cap, char *arch,
+                               int32_t arch_cap, int32_t *n_cu, int32_t *clock_khz,
+                               int32_t *mem_clock_khz, int64_t *mem_bytes);
+
+/* alloc_zeros::<T>(n), src/cuda.rs:723,757,926,1052,1066: zero-filled device memory. */
+int32_t galois_hip_alloc_zeros(galois_hip_ctx *ctx, size_t bytes, void **out);
+/* Drop of CudaSlice<T>. */
+int32_t galois_hip_free(galois_hip_ctx *ctx, void *dptr);
+/* htod_sync_copy, src/cuda.rs:234,250,274,281,288. */
+int32_t galois_hip_htod_sync_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+/* dtoh_sync_copy_into, src/lib.rs:2217-2328: waits for the stream, then copies. */
+int32_t galois_hip_dtoh_sync_copy(galois_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+/* cudaMemcpyAsync / cudaMemcpy2DAsync device-to-device, src/cuda.rs:335-371 (pitches in bytes). */
+int32_t galois_hip_dtod_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
+int32_t galois_hip_dtod_copy_2d(galois_hip_ctx *ctx, void *dst_dev, size_t dpitch, const void *src_dev,
+                                size_t spitch, size_t width_bytes, size_t height);
+/* Stream synchronisation (implicit in the reference's to_cpu_tensor, src/lib.rs:2314). */
+int32_t galois_hip_synchronize(galois_hip_ctx *ctx);
+
+/* Timing on the context's stream (the reference has none: dead SystemTime pairs, src/op.rs:1392-1395). */
+int32_t galois_hip_event_create(galois_hip_ctx *ctx, galois_hip_event **out);
+int32_t galois_hip_event_record(galois_hip_ctx *ctx, galois_hip_event *ev);
+int32_t galois_hip_event_elapsed_ms(galois_hip_ctx *ctx, galois_hip_event *start, galois_hip_event *stop,
+                                    float *ms); /* synchronises on `stop` */
+int32_t galois_hip_event_destroy(galois_hip_ctx *ctx, galois_hip_event *ev);
+
+/* ---- the hot path --------------------------------------------------------- */
+
+/* Decode GEMV.  Replaces the launch of dequantize_mul_mat_vec_q4_0
+ * (src/cuda.rs:1011-1034 -> galois-kernels/src/matmul.cu:45-117), same argument
+ * order: dst[row] = sum_col (q-8)*d * y[col], f32.  vx: nrows rows of ncols/32
+ * Q4_0 blocks; ncols % 32 == 0; vx 2-byte aligned, y/dst 4-byte aligned.
+ * The caller loops ne12*ne13 batch slices exactly as src/cuda.rs:1026-1034. */
+int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, const void *vx, const float *y,
+                                               float *dst, int32_t ncols, int32_t nrows);
+
+/* Prefill matmul.  Replaces quantize_q8_1 + mul_mat_q4_0 (src/cuda.rs:1035-1136 ->
+ * matmul.cu:133-174,452-504) with one call: Y[m*N + n] = sum_k deq(W)[n,k] * X[m*K + k]
+ * (output layout of matmul.cu:359).  W tiles are dequantised to fp16 in LDS, X is
+ * rounded to fp16, products accumulate in f32 on MFMA.  K % 32 == 0.  No Q8_1
+ * scratch and no K padding (src/cuda.rs:1040-1068) are needed. */
+int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *W, const float *X, float *Y,
+                                    int32_t K, int32_t N, int32_t M);
+
+/* rms_norm_f32 launch, src/cuda.rs:1146-1181 -> rms_norm.cu:13-49:
+ * dst = x * rsqrt(mean(x^2) + eps) per row.  Unlike the reference (ne00 % 32 == 0
+ * asserted at src/cuda.rs:1157) any ncols >= 1 is accepted. */
+int32_t galois_hip_rms_norm_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols,
+                                int32_t nrows, float eps);
+/* Fusion of rms_norm_f32 with the broadcast mul_f32 that applies the norm weight
+ * (src/cuda.rs:1190-1215 -> mul.cu:3-12): dst = rms_norm(x) * weight[col]. */
+int32_t galois_hip_rms_norm_mul_f32(galois_hip_ctx *ctx, const float *x, const float *weight, float *dst,
+                                    int32_t ncols, int32_t nrows, float eps);
+
+/* rope_f32 launch, src/cuda.rs:1257-1297 -> rope.cu:3-28, same parameters (has_pos is
+ * always true in the reference): adjacent pairs rotated by
+ * pos[row / p_delta_rows] * freq_scale * theta_scale^(col/2).  ncols even. */
+int32_t galois_hip_rope_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols, int32_t nrows,
+                            const int32_t *pos, float freq_scale, int32_t p_delta_rows, float theta_scale);
+
+/* soft_max_f32 launch, src/cuda.rs:1642-1663 -> softmax.cu:3-48: row softmax in f32,
+ * -inf inputs are masked (exactly 0 out).  A row that is all -inf yields NaN as in the
+ * reference kernel. */
+int32_t galois_hip_soft_max_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols,
+                                int32_t nrows);
+/* Causal variant with the mask computed from indices instead of -inf inputs (the
+ * reference has no mask op): row r keeps columns <= n_past + (r % rows_per_head),
+ * other outputs are exactly 0 and their inputs are never read. */
+int32_t galois_hip_soft_max_causal_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols,
+                                       int32_t rows_per_head, int32_t nrows, int32_t n_past);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GALOIS_HIP_H */
