@@ -143,6 +143,12 @@ class Device:
         self._check(self._lib.galois_hip_event_destroy(self._ctx, ev))
 
     # -- ops: same argument order as the C ABI ----------------------------------------
+    def quantize_row_q4_0(self, x, y, k):
+        self._check(self._lib.galois_hip_quantize_row_q4_0(self._ctx, _ptr(x), _ptr(y), k))
+
+    def dequantize_row_q4_0(self, x, y, k):
+        self._check(self._lib.galois_hip_dequantize_row_q4_0(self._ctx, _ptr(x), _ptr(y), k))
+
     def dequantize_mul_mat_vec_q4_0(self, vx, y, dst, ncols, nrows):
         self._check(self._lib.galois_hip_dequantize_mul_mat_vec_q4_0(self._ctx, _ptr(vx), _ptr(y), _ptr(dst),
                                                                      ncols, nrows))

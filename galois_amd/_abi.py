@@ -32,6 +32,8 @@ PROTOTYPES = {
     "galois_hip_event_record": (i32, [c_ctx, c_ev]),
     "galois_hip_event_elapsed_ms": (i32, [c_ctx, c_ev, c_ev, C.POINTER(f32)]),
     "galois_hip_event_destroy": (i32, [c_ctx, c_ev]),
+    "galois_hip_quantize_row_q4_0": (i32, [c_ctx, vp, vp, C.c_int64]),
+    "galois_hip_dequantize_row_q4_0": (i32, [c_ctx, vp, vp, C.c_int64]),
     "galois_hip_dequantize_mul_mat_vec_q4_0": (i32, [c_ctx, vp, vp, vp, i32, i32]),
     "galois_hip_mul_mat_q4_0_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32]),
     "galois_hip_rms_norm_f32": (i32, [c_ctx, vp, vp, i32, i32, f32]),

@@ -86,6 +86,17 @@ int32_t galois_hip_event_elapsed_ms(galois_hip_ctx *ctx, galois_hip_event *start
                                     float *ms); /* synchronises on `stop` */
 int32_t galois_hip_event_destroy(galois_hip_ctx *ctx, galois_hip_event *ev);
 
+/* ---- Q4_0 format ----------------------------------------------------------- */
+
+/* BlockQ4_0::from_f32 is todo!() in the reference (src/ggml_quants.rs:198-200); this is the
+ * canonical ggml quantize_row_q4_0 whose output BlockQ4_0::to_f32 (src/ggml_quants.rs:209-228)
+ * inverts: k floats -> k/32 blocks of 18 bytes.  k % 32 == 0.  Rows of a matrix are
+ * quantized by one call over the whole contiguous buffer (blocks never straddle rows when
+ * the row length is a multiple of 32). */
+int32_t galois_hip_quantize_row_q4_0(galois_hip_ctx *ctx, const float *x, void *y, int64_t k);
+/* BlockQ4_0::to_f32, src/ggml_quants.rs:209-228 (device twin dequantize_q4_0, matmul.cu:25-43). */
+int32_t galois_hip_dequantize_row_q4_0(galois_hip_ctx *ctx, const void *x, float *y, int64_t k);
+
 /* ---- the hot path --------------------------------------------------------- */
 
 /* Decode GEMV.  Replaces the launch of dequantize_mul_mat_vec_q4_0
