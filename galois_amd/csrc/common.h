@@ -12,6 +12,8 @@ struct galois_hip_ctx {
     hipStream_t stream;
     int32_t n_cu;
     int32_t gemv_config;  // 0 = choose from the shape; GALOIS_HIP_GEMV_CONFIG=1..5 forces a kernel shape (tuning)
+    void *ws;         // workspace owned by the context (fp16 activations of the prefill matmul)
+    size_t ws_bytes;
     char last_error[256];
 };
 

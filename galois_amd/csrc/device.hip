@@ -36,6 +36,8 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     ctx->ordinal = ordinal;
     ctx->n_cu = prop.multiProcessorCount;
     ctx->last_error[0] = 0;
+    ctx->ws = nullptr;
+    ctx->ws_bytes = 0;
     const char *cfg = getenv("GALOIS_HIP_GEMV_CONFIG");
     ctx->gemv_config = cfg ? atoi(cfg) : 0;
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
@@ -51,6 +53,7 @@ int32_t galois_hip_destroy(galois_hip_ctx *ctx) {
     GH_REQUIRE_CTX(ctx);
     (void)hipSetDevice(ctx->ordinal);
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->ws) (void)hipFree(ctx->ws);
     hipError_t e = hipStreamDestroy(ctx->stream);
     delete ctx;
     return (int32_t)e;
