@@ -34,6 +34,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 MFMA, published
 GEMV_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000)]  # (K, N)
 PREFILL = (512, 4096, 11008)    # (M, K, N)
 ROTATE_BYTES = 1200 << 20
+# HBM bytes per GEMV launch (average over the four shapes) measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE on this workload, each scaled by what the same counter reads for a device-to-device copy of
+# known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); see profiles/gemv_q4_0_dot8__llama7b_gemv_set.md
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 33779200
 
 
 def q4_bytes(k, n):
@@ -205,7 +209,8 @@ def main():
                                "K11008->N4096, K4096->N32000 (BASELINE.json configs[1])",
                    "weight_bytes_per_step": set_bytes, "launches_per_step": launches},
         "roofline": {"bound": "hbm", "achieved": round(avg_bytes / avg_us / 1e3, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(avg_bytes / avg_us / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(avg_bytes / avg_us / 1e3 / HBM_PEAK_GBPS, 4),
+                     "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "gemv_q4_0_dot8", "bytes_per_launch": avg_bytes, "us_per_launch": round(avg_us, 3)},
     }
     if not args.no_cpu:
