@@ -39,7 +39,22 @@ def build(verbose=False, extra=()):
     subprocess.check_call(cmd)
     if verbose:
         print("built", LIB)
+    build_host(verbose)
     return LIB
+
+
+HOST_LIB = os.path.join(HERE, "libgalois_host.so")
+
+
+def build_host(verbose=False):
+    """The C++ host mirror of galois's op layer (g++ only: it sees nothing but include/galois_hip.h)."""
+    srcs = sorted(glob.glob(os.path.join(HERE, "host", "*.cpp")))
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", HOST_LIB, *srcs,
+           "-L" + HERE, "-lgalois_hip", "-Wl,-rpath,$ORIGIN"]
+    subprocess.check_call(cmd)
+    if verbose:
+        print("built", HOST_LIB)
+    return HOST_LIB
 
 
 if __name__ == "__main__":

@@ -1,0 +1,143 @@
+"""ctypes face of libgalois_host.so, the C++ mirror of galois's Tensor / op interface.
+
+Names follow the reference: ``Tensor.from_raw`` (src/lib.rs:2477), ``to_cpu_tensor``
+(src/lib.rs:2279), ``galois_matmul`` / ``galois_rms_norm`` / ``galois_rope_custom`` /
+``galois_soft_max`` (src/op.rs:3093-3341).  Shapes are ggml order: ne0 (innermost) first.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libgalois_host.so")
+
+F32, F16, Q4_0, I32 = 0, 1, 2, 18
+_NP = {F32: np.float32, F16: np.float16, Q4_0: np.uint8, I32: np.int32}
+KINDS = {1: "Unimplemented", 2: "ShapeError", 3: "DeviceError", 4: "Unexpected"}
+
+
+class GError(RuntimeError):
+    def __init__(self, kind, msg):
+        super().__init__("%s: %s" % (KINDS.get(kind, kind), msg))
+        self.kind = KINDS.get(kind, kind)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("galois_amd: %s is missing -- build with `python -m galois_amd.build`" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        vp, sz = C.c_void_p, C.c_size_t
+        L.galois_host_last_error.restype = C.c_char_p
+        for name, res, args in (
+                ("galois_host_device_new", vp, [C.c_int]), ("galois_host_device_cpu", vp, []),
+                ("galois_host_device_free", None, [vp]),
+                ("galois_host_tensor_from_raw", vp, [vp, vp, sz, sz, C.POINTER(sz), C.c_int]),
+                ("galois_host_tensor_zeros", vp, [vp, sz, C.POINTER(sz), C.c_int]),
+                ("galois_host_tensor_view", vp, [vp, sz, sz, C.POINTER(sz)]),
+                ("galois_host_tensor_to_cpu", C.c_int, [vp, vp, sz]), ("galois_host_tensor_nbytes", sz, [vp]),
+                ("galois_host_tensor_free", None, [vp]), ("galois_host_matmul", C.c_int, [vp, vp, vp]),
+                ("galois_host_rms_norm", C.c_int, [vp, vp, C.c_float]),
+                ("galois_host_rope_custom", C.c_int, [sz, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int,
+                                                      vp, vp, vp]),
+                ("galois_host_soft_max", C.c_int, [vp, vp])):
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _raise(kind=4):
+    raise GError(kind, lib().galois_host_last_error().decode())
+
+
+def _shape(shape):
+    return len(shape), (C.c_size_t * len(shape))(*shape)
+
+
+class Device:
+    """``Device::Cpu`` or ``Device::Gpu(CudaDevice::new(ordinal))``."""
+
+    def __init__(self, h):
+        self.h = h
+
+    @staticmethod
+    def cpu():
+        return Device(lib().galois_host_device_cpu())
+
+    @staticmethod
+    def gpu(ordinal=0):
+        h = lib().galois_host_device_new(ordinal)
+        if not h:
+            _raise(3)
+        return Device(h)
+
+
+class Tensor:
+    def __init__(self, h, shape, dtype):
+        self.h, self.shape, self.dtype = h, tuple(shape), dtype
+
+    @staticmethod
+    def from_raw(data, shape, dtype, device):
+        """``Tensor::from_raw(bytes, n_dims, Shape::from_array(shape), dtype, &device)``."""
+        data = np.ascontiguousarray(data)
+        n, s = _shape(shape)
+        h = lib().galois_host_tensor_from_raw(device.h, data.ctypes.data_as(C.c_void_p), data.nbytes, n, s, dtype)
+        if not h:
+            _raise(2)
+        return Tensor(h, shape, dtype)
+
+    @staticmethod
+    def zeros(shape, dtype, device):
+        n, s = _shape(shape)
+        h = lib().galois_host_tensor_zeros(device.h, n, s, dtype)
+        if not h:
+            _raise(2)
+        return Tensor(h, shape, dtype)
+
+    def view(self, elem_offset, shape):
+        n, s = _shape(shape)
+        h = lib().galois_host_tensor_view(self.h, elem_offset, n, s)
+        if not h:
+            _raise(2)
+        return Tensor(h, shape, self.dtype)
+
+    def to_cpu_tensor(self):
+        """Host copy as a numpy array shaped [ne3..ne0] (row-major), uint8 block bytes for Q4_0."""
+        nb = lib().galois_host_tensor_nbytes(self.h)
+        out = np.empty(nb, np.uint8)
+        st = lib().galois_host_tensor_to_cpu(self.h, out.ctypes.data_as(C.c_void_p), nb)
+        if st:
+            _raise(st)
+        if self.dtype == Q4_0:
+            return out
+        return out.view(_NP[self.dtype]).reshape(tuple(reversed(self.shape)))
+
+
+def _call(st):
+    if st:
+        _raise(st)
+
+
+def galois_matmul(a, b, dst):
+    _call(lib().galois_host_matmul(a.h, b.h, dst.h))
+
+
+def galois_rms_norm(src, dst, eps):
+    _call(lib().galois_host_rms_norm(src.h, dst.h, eps))
+
+
+def galois_rope_custom(op, src0, src1, dst):
+    _call(lib().galois_host_rope_custom(op["n_dims"], op.get("mode", 0), op.get("n_ctx", 0),
+                                        op.get("freq_base", 10000.0), op.get("freq_scale", 1.0),
+                                        op.get("xpos_base", 0.0), int(op.get("xpos_down", False)), src0.h, src1.h,
+                                        dst.h))
+
+
+def galois_soft_max(src, dst):
+    _call(lib().galois_host_soft_max(src.h, dst.h))

@@ -74,3 +74,23 @@ def test_product_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".hpp", ".cpp", ".c")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_host_mirror_builds_and_uses_only_the_c_abi():
+    """libgalois_host.so (C++ mirror of galois's op layer) links against libgalois_hip.so and nothing of HIP."""
+    from galois_amd import host_api
+    assert os.path.exists(host_api.LIB_PATH), "build first: python -m galois_amd.build"
+    host_api.lib()
+    out = subprocess.check_output(["nm", "-D", "--undefined-only", host_api.LIB_PATH], text=True)
+    used = sorted(set(re.findall(r"\bgalois_hip_[a-z0-9_]+", out)))
+    assert "galois_hip_dequantize_mul_mat_vec_q4_0" in used and "galois_hip_mul_mat_q4_0_f32" in used
+    assert set(used) <= set(_declared())
+    assert not re.search(r"\bhip[A-Z]", out), "the host mirror must not call HIP directly"
+    # CPU tensors work without a GPU; GPU ops on them are 'Unimplemented', never a crash
+    import numpy as np
+    cpu = host_api.Device.cpu()
+    t = host_api.Tensor.from_raw(np.arange(8, dtype=np.float32), [4, 2], host_api.F32, cpu)
+    assert np.array_equal(t.to_cpu_tensor(), np.arange(8, dtype=np.float32).reshape(2, 4))
+    with pytest.raises(host_api.GError) as e:
+        host_api.galois_soft_max(t, t)
+    assert e.value.kind == "Unimplemented"
