@@ -173,3 +173,29 @@ class Device:
     def soft_max_causal_f32(self, x, dst, ncols, rows_per_head, nrows, n_past):
         self._check(self._lib.galois_hip_soft_max_causal_f32(self._ctx, _ptr(x), _ptr(dst), ncols, rows_per_head,
                                                              nrows, n_past))
+
+    def add_f32(self, x, y, dst, kx, ky):
+        self._check(self._lib.galois_hip_add_f32(self._ctx, _ptr(x), _ptr(y), _ptr(dst), kx, ky))
+
+    def mul_f32(self, x, y, dst, kx, ky):
+        self._check(self._lib.galois_hip_mul_f32(self._ctx, _ptr(x), _ptr(y), _ptr(dst), kx, ky))
+
+    def scale_f32(self, x, dst, scale, k):
+        self._check(self._lib.galois_hip_scale_f32(self._ctx, _ptr(x), _ptr(dst), scale, k))
+
+    def silu_f32(self, x, dst, k):
+        self._check(self._lib.galois_hip_silu_f32(self._ctx, _ptr(x), _ptr(dst), k))
+
+    def silu_mul_f32(self, gate, up, dst, k):
+        self._check(self._lib.galois_hip_silu_mul_f32(self._ctx, _ptr(gate), _ptr(up), _ptr(dst), k))
+
+    def cpy_f32(self, x, dst, dst_is_f16, ne, ne00, ne01, nb00, nb01, nb02, ne10, ne11, nb10, nb11, nb12):
+        self._check(self._lib.galois_hip_cpy_f32(self._ctx, _ptr(x), _ptr(dst), int(dst_is_f16), ne, ne00, ne01, nb00,
+                                                 nb01, nb02, ne10, ne11, nb10, nb11, nb12))
+
+    def get_rows_q4_0(self, table, ids, dst, ncols, nr):
+        self._check(self._lib.galois_hip_get_rows_q4_0(self._ctx, _ptr(table), _ptr(ids), _ptr(dst), ncols, nr))
+
+    def mul_mat_f32(self, a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2):
+        self._check(self._lib.galois_hip_mul_mat_f32(self._ctx, _ptr(a), _ptr(b), _ptr(dst), K, N, M, ne02, ne12,
+                                                     a_s0, a_s1, a_s2))

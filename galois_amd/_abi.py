@@ -41,6 +41,14 @@ PROTOTYPES = {
     "galois_hip_rope_f32": (i32, [c_ctx, vp, vp, i32, i32, vp, f32, i32, f32]),
     "galois_hip_soft_max_f32": (i32, [c_ctx, vp, vp, i32, i32]),
     "galois_hip_soft_max_causal_f32": (i32, [c_ctx, vp, vp, i32, i32, i32, i32]),
+    "galois_hip_add_f32": (i32, [c_ctx, vp, vp, vp, C.c_int64, C.c_int64]),
+    "galois_hip_mul_f32": (i32, [c_ctx, vp, vp, vp, C.c_int64, C.c_int64]),
+    "galois_hip_scale_f32": (i32, [c_ctx, vp, vp, f32, C.c_int64]),
+    "galois_hip_silu_f32": (i32, [c_ctx, vp, vp, C.c_int64]),
+    "galois_hip_silu_mul_f32": (i32, [c_ctx, vp, vp, vp, C.c_int64]),
+    "galois_hip_cpy_f32": (i32, [c_ctx, vp, vp, i32] + [C.c_int64] * 11),
+    "galois_hip_get_rows_q4_0": (i32, [c_ctx, vp, vp, vp, i32, i32]),
+    "galois_hip_mul_mat_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32, i32, i32, C.c_int64, C.c_int64, C.c_int64]),
 }
 
 _lib = None

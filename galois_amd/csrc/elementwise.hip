@@ -1,0 +1,275 @@
+// Elementwise, copy and gather kernels around the Q4_0 path (the reference's add / mul / scale /
+// silu / cpy kernels and the CPU-only get_rows), plus the f32 batched matmul the attention of a
+// decode step needs.  All are HBM-bound, one read and one write per element.
+#include "common.h"
+
+namespace {
+
+constexpr int kEwThreads = 256;
+
+enum { EW_ADD = 0, EW_MUL = 1 };
+
+// add_f32 / mul_f32 (galois-kernels/src/add.cu:3-12, mul.cu:3-12): dst[i] = x[i] op y[i % ky].
+// The reference launcher swaps grid and block (src/cuda.rs:1206-1210, 1235-1239); not copied.
+template <int OP>
+__global__ __launch_bounds__(kEwThreads) void ew_bcast(const float *__restrict__ x, const float *__restrict__ y,
+                                                       float *__restrict__ dst, int64_t kx, int64_t ky) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i >= kx) return;
+    const float b = y[i % ky];
+    dst[i] = OP == EW_ADD ? x[i] + b : x[i] * b;
+}
+
+// Vector form when kx, ky are multiples of 4 and pointers 16-byte aligned: y index never splits a float4.
+template <int OP>
+__global__ __launch_bounds__(kEwThreads) void ew_bcast4(const float4 *__restrict__ x, const float4 *__restrict__ y,
+                                                        float4 *__restrict__ dst, int64_t kx4, int64_t ky4) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i >= kx4) return;
+    const float4 a = x[i], b = y[i % ky4];
+    dst[i] = OP == EW_ADD ? make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w)
+                          : make_float4(a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w);
+}
+
+// scale_f32 (scale.cu:1-11)
+__global__ __launch_bounds__(kEwThreads) void ew_scale(const float *__restrict__ x, float *__restrict__ dst,
+                                                       float scale, int64_t k) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i < k) dst[i] = scale * x[i];
+}
+
+// silu_f32 (unary.cu:1-10): x / (1 + exp(-x)); with `up` != nullptr the SwiGLU product silu(x) * up.
+__global__ __launch_bounds__(kEwThreads) void ew_silu(const float *__restrict__ x, const float *__restrict__ up,
+                                                      float *__restrict__ dst, int64_t k) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i >= k) return;
+    const float v = x[i];
+    const float s = v / (1.0f + expf(-v));
+    dst[i] = up ? s * up[i] : s;
+}
+
+// cpy_f32_f32 / cpy_f32_f16 (cpy.cu:79-156): element i of a [ne00, ne01, *] source with byte
+// strides nb00.. is written to element i of a [ne10, ne11, *] destination with byte strides nb10..
+template <typename DST>
+__global__ __launch_bounds__(kEwThreads) void cpy_strided(const char *__restrict__ cx, char *__restrict__ cdst,
+                                                          int64_t ne, int64_t ne00, int64_t ne01, int64_t nb00,
+                                                          int64_t nb01, int64_t nb02, int64_t ne10, int64_t ne11,
+                                                          int64_t nb10, int64_t nb11, int64_t nb12) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i >= ne) return;
+    const int64_t i02 = i / (ne00 * ne01), r0 = i - i02 * ne00 * ne01;
+    const int64_t i01 = r0 / ne00, i00 = r0 - i01 * ne00;
+    const int64_t i12 = i / (ne10 * ne11), r1 = i - i12 * ne10 * ne11;
+    const int64_t i11 = r1 / ne10, i10 = r1 - i11 * ne10;
+    const float v = *reinterpret_cast<const float *>(cx + i00 * nb00 + i01 * nb01 + i02 * nb02);
+    *reinterpret_cast<DST *>(cdst + i10 * nb10 + i11 * nb11 + i12 * nb12) = (DST)v;
+}
+
+// get_rows for a Q4_0 table (GetRows::f_q_x_f32, src/op.rs:2546-2571; CPU-only in the reference):
+// dst row i = to_f32(table row ids[i]).  One wave per row, one block per lane per step.
+__global__ __launch_bounds__(kEwThreads) void get_rows_q4_0(const uint16_t *__restrict__ table,
+                                                            const int32_t *__restrict__ ids, float *__restrict__ dst,
+                                                            int nblocks, int nr) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
+    if (r >= nr) return;
+    const uint16_t *row = table + (size_t)ids[r] * nblocks * 9;
+    float *out = dst + (size_t)r * nblocks * 32;
+    for (int b = lane; b < nblocks; b += 64) {
+        const uint16_t *p = row + (size_t)b * 9;
+        const float d = (float)__builtin_bit_cast(_Float16, p[0]);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t v = p[1 + j];
+            out[b * 32 + 2 * j] = (float)((int)(v & 0xF) - 8) * d;
+            out[b * 32 + 2 * j + 16] = (float)((int)((v >> 4) & 0xF) - 8) * d;
+            out[b * 32 + 2 * j + 1] = (float)((int)((v >> 8) & 0xF) - 8) * d;
+            out[b * 32 + 2 * j + 17] = (float)((int)((v >> 12) & 0xF) - 8) * d;
+        }
+    }
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_mov<0xB1>(v);
+    v += dpp_mov<0x4E>(v);
+    v += dpp_mov<0x141>(v);
+    v += dpp_mov<0x140>(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// f32 x f32 batched matmul, rows of `a` contiguous along K (a_s0 == 1): dst[i2][m][n] =
+// sum_k a[(i2/r2)*a_s2 + n*a_s1 + k] * b[(i2*M + m)*K + k].  One wave per (n, i2); the QK^T of
+// a decode step (K = head_dim, N = cached positions).
+__global__ __launch_bounds__(kEwThreads) void mul_mat_f32_krows(const float *__restrict__ a,
+                                                                const float *__restrict__ b, float *__restrict__ dst,
+                                                                int K, int N, int M, int r2, int64_t a_s1,
+                                                                int64_t a_s2) {
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
+    const int i2 = blockIdx.y;
+    if (n >= N) return;
+    const float *ar = a + (int64_t)(i2 / r2) * a_s2 + (int64_t)n * a_s1;
+    for (int m = 0; m < M; m++) {
+        const float *br = b + ((int64_t)i2 * M + m) * K;
+        float acc = 0.0f;
+        for (int k = lane; k < K; k += 64) acc = __builtin_fmaf(ar[k], br[k], acc);
+        acc = wave_sum(acc);
+        if (lane == 0) dst[((int64_t)i2 * M + m) * N + n] = acc;
+    }
+}
+
+// Same contraction when `a` is contiguous along N (a_s1 == 1, K strided by a_s0): the P.V of a
+// decode step (K = cached positions, N = head_dim).  A workgroup owns 64 columns n of one batch
+// slice; its 4 waves split K and combine through LDS.
+__global__ __launch_bounds__(kEwThreads) void mul_mat_f32_ncols(const float *__restrict__ a,
+                                                                const float *__restrict__ b, float *__restrict__ dst,
+                                                                int K, int N, int M, int r2, int64_t a_s0,
+                                                                int64_t a_s2) {
+    __shared__ float part[kEwThreads];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + lane;
+    const int i2 = blockIdx.y;
+    const float *ab = a + (int64_t)(i2 / r2) * a_s2;
+    for (int m = 0; m < M; m++) {
+        const float *br = b + ((int64_t)i2 * M + m) * K;
+        float acc = 0.0f;
+        if (n < N)
+            for (int k = wave; k < K; k += kEwThreads / 64) acc = __builtin_fmaf(ab[(int64_t)k * a_s0 + n], br[k], acc);
+        part[threadIdx.x] = acc;
+        __syncthreads();
+        if (wave == 0 && n < N)
+            dst[((int64_t)i2 * M + m) * N + n] = (part[lane] + part[64 + lane]) + (part[128 + lane] + part[192 + lane]);
+        __syncthreads();
+    }
+}
+
+int32_t launch_bcast(galois_hip_ctx *ctx, int op, const float *x, const float *y, float *dst, int64_t kx, int64_t ky,
+                     const char *what) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && y && dst, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, kx > 0 && ky > 0 && kx <= (int64_t)0x7FFFFFFF * kEwThreads, GALOIS_HIP_E_SHAPE, what);
+    GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(y, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, what);
+    GH_BIND(ctx);
+    if (kx % 4 == 0 && ky % 4 == 0 && gh_aligned(x, 16) && gh_aligned(y, 16) && gh_aligned(dst, 16)) {
+        const dim3 grid((unsigned)((kx / 4 + kEwThreads - 1) / kEwThreads));
+        if (op == EW_ADD)
+            hipLaunchKernelGGL(ew_bcast4<EW_ADD>, grid, dim3(kEwThreads), 0, ctx->stream, (const float4 *)x,
+                               (const float4 *)y, (float4 *)dst, kx / 4, ky / 4);
+        else
+            hipLaunchKernelGGL(ew_bcast4<EW_MUL>, grid, dim3(kEwThreads), 0, ctx->stream, (const float4 *)x,
+                               (const float4 *)y, (float4 *)dst, kx / 4, ky / 4);
+    } else {
+        const dim3 grid((unsigned)((kx + kEwThreads - 1) / kEwThreads));
+        if (op == EW_ADD)
+            hipLaunchKernelGGL(ew_bcast<EW_ADD>, grid, dim3(kEwThreads), 0, ctx->stream, x, y, dst, kx, ky);
+        else
+            hipLaunchKernelGGL(ew_bcast<EW_MUL>, grid, dim3(kEwThreads), 0, ctx->stream, x, y, dst, kx, ky);
+    }
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t galois_hip_add_f32(galois_hip_ctx *ctx, const float *x, const float *y, float *dst, int64_t kx, int64_t ky) {
+    return launch_bcast(ctx, EW_ADD, x, y, dst, kx, ky, "add_f32");
+}
+
+int32_t galois_hip_mul_f32(galois_hip_ctx *ctx, const float *x, const float *y, float *dst, int64_t kx, int64_t ky) {
+    return launch_bcast(ctx, EW_MUL, x, y, dst, kx, ky, "mul_f32");
+}
+
+int32_t galois_hip_scale_f32(galois_hip_ctx *ctx, const float *x, float *dst, float scale, int64_t k) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && dst, GALOIS_HIP_E_NULL, "scale_f32");
+    GH_REQUIRE(ctx, k > 0 && k <= (int64_t)0x7FFFFFFF * kEwThreads, GALOIS_HIP_E_SHAPE, "scale_f32");
+    GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "scale_f32");
+    GH_BIND(ctx);
+    hipLaunchKernelGGL(ew_scale, dim3((unsigned)((k + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0, ctx->stream,
+                       x, dst, scale, k);
+    GH_LAUNCH_CHECK(ctx, "scale_f32 launch");
+}
+
+static int32_t launch_silu(galois_hip_ctx *ctx, const float *x, const float *up, float *dst, int64_t k,
+                           const char *what) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && dst, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, k > 0 && k <= (int64_t)0x7FFFFFFF * kEwThreads, GALOIS_HIP_E_SHAPE, what);
+    GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(up, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, what);
+    GH_BIND(ctx);
+    hipLaunchKernelGGL(ew_silu, dim3((unsigned)((k + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0, ctx->stream,
+                       x, up, dst, k);
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
+int32_t galois_hip_silu_f32(galois_hip_ctx *ctx, const float *x, float *dst, int64_t k) {
+    return launch_silu(ctx, x, nullptr, dst, k, "silu_f32");
+}
+
+int32_t galois_hip_silu_mul_f32(galois_hip_ctx *ctx, const float *gate, const float *up, float *dst, int64_t k) {
+    if (ctx && !up) return gh_fail(ctx, GALOIS_HIP_E_NULL, "silu_mul_f32: up");
+    return launch_silu(ctx, gate, up, dst, k, "silu_mul_f32");
+}
+
+int32_t galois_hip_cpy_f32(galois_hip_ctx *ctx, const void *x, void *dst, int32_t dst_is_f16, int64_t ne, int64_t ne00,
+                           int64_t ne01, int64_t nb00, int64_t nb01, int64_t nb02, int64_t ne10, int64_t ne11,
+                           int64_t nb10, int64_t nb11, int64_t nb12) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, x && dst, GALOIS_HIP_E_NULL, "cpy_f32");
+    GH_REQUIRE(ctx, ne > 0 && ne00 > 0 && ne01 > 0 && ne10 > 0 && ne11 > 0 && ne <= (int64_t)0x7FFFFFFF * kEwThreads,
+               GALOIS_HIP_E_SHAPE, "cpy_f32");
+    const int64_t dsz = dst_is_f16 ? 2 : 4;
+    GH_REQUIRE(ctx, nb00 % 4 == 0 && nb01 % 4 == 0 && nb02 % 4 == 0 && nb10 % dsz == 0 && nb11 % dsz == 0 &&
+                        nb12 % dsz == 0 && gh_aligned(x, 4) && gh_aligned(dst, (size_t)dsz),
+               GALOIS_HIP_E_ALIGN, "cpy_f32: strides and pointers must be multiples of the element size");
+    GH_BIND(ctx);
+    const dim3 grid((unsigned)((ne + kEwThreads - 1) / kEwThreads));
+    if (dst_is_f16)
+        hipLaunchKernelGGL(cpy_strided<_Float16>, grid, dim3(kEwThreads), 0, ctx->stream, (const char *)x, (char *)dst,
+                           ne, ne00, ne01, nb00, nb01, nb02, ne10, ne11, nb10, nb11, nb12);
+    else
+        hipLaunchKernelGGL(cpy_strided<float>, grid, dim3(kEwThreads), 0, ctx->stream, (const char *)x, (char *)dst, ne,
+                           ne00, ne01, nb00, nb01, nb02, ne10, ne11, nb10, nb11, nb12);
+    GH_LAUNCH_CHECK(ctx, "cpy_f32 launch");
+}
+
+int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const int32_t *ids, float *dst, int32_t ncols,
+                                 int32_t nr) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, table && ids && dst, GALOIS_HIP_E_NULL, "get_rows_q4_0");
+    GH_REQUIRE(ctx, ncols > 0 && ncols % 32 == 0 && nr > 0, GALOIS_HIP_E_SHAPE, "get_rows_q4_0");
+    GH_REQUIRE(ctx, gh_aligned(table, 2) && gh_aligned(ids, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "get_rows_q4_0");
+    GH_BIND(ctx);
+    hipLaunchKernelGGL(get_rows_q4_0, dim3((nr + 3) / 4), dim3(kEwThreads), 0, ctx->stream, (const uint16_t *)table,
+                       ids, dst, ncols / 32, nr);
+    GH_LAUNCH_CHECK(ctx, "get_rows_q4_0 launch");
+}
+
+int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K, int32_t N,
+                               int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, a && b && dst, GALOIS_HIP_E_NULL, "mul_mat_f32");
+    GH_REQUIRE(ctx, K > 0 && N > 0 && M > 0 && ne02 > 0 && ne12 > 0 && ne12 % ne02 == 0 && ne12 <= 65535,
+               GALOIS_HIP_E_SHAPE, "mul_mat_f32");
+    GH_REQUIRE(ctx, a_s0 == 1 || a_s1 == 1, GALOIS_HIP_E_UNSUPPORTED,
+               "mul_mat_f32: a must be contiguous along K (a_s0 == 1) or along N (a_s1 == 1)");
+    GH_REQUIRE(ctx, gh_aligned(a, 4) && gh_aligned(b, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "mul_mat_f32");
+    GH_BIND(ctx);
+    const int r2 = ne12 / ne02;
+    if (a_s0 == 1)
+        hipLaunchKernelGGL(mul_mat_f32_krows, dim3((N + 3) / 4, ne12), dim3(kEwThreads), 0, ctx->stream, a, b, dst, K, N,
+                           M, r2, a_s1, a_s2);
+    else
+        hipLaunchKernelGGL(mul_mat_f32_ncols, dim3((N + 63) / 64, ne12), dim3(kEwThreads), 0, ctx->stream, a, b, dst, K,
+                           N, M, r2, a_s0, a_s2);
+    GH_LAUNCH_CHECK(ctx, "mul_mat_f32 launch");
+}
+
+}  // extern "C"

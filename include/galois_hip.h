@@ -142,6 +142,36 @@ int32_t galois_hip_soft_max_f32(galois_hip_ctx *ctx, const float *x, float *dst,
 int32_t galois_hip_soft_max_causal_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols,
                                        int32_t rows_per_head, int32_t nrows, int32_t n_past);
 
+/* ---- around the hot path: the other ops of a LLaMA decode graph --------------------- */
+
+/* add_f32 / mul_f32, src/cuda.rs:1188-1244 -> add.cu:3-12, mul.cu:3-12: dst[i] = x[i] (op) y[i % ky]
+ * (row broadcast of a bias / norm weight; ky == kx is the plain elementwise case). */
+int32_t galois_hip_add_f32(galois_hip_ctx *ctx, const float *x, const float *y, float *dst, int64_t kx, int64_t ky);
+int32_t galois_hip_mul_f32(galois_hip_ctx *ctx, const float *x, const float *y, float *dst, int64_t kx, int64_t ky);
+/* scale_f32, src/cuda.rs:1597-1638 -> scale.cu:1-11: dst = scale * x (the caller reads the scalar
+ * out of its CPU tensor as CudaScale::f_g_c does). */
+int32_t galois_hip_scale_f32(galois_hip_ctx *ctx, const float *x, float *dst, float scale, int64_t k);
+/* silu_f32, src/cuda.rs:1665-1688 -> unary.cu:1-10: dst = x / (1 + exp(-x)). */
+int32_t galois_hip_silu_f32(galois_hip_ctx *ctx, const float *x, float *dst, int64_t k);
+/* Fusion of silu_f32 with the elementwise mul_f32 of SwiGLU: dst = silu(gate) * up. */
+int32_t galois_hip_silu_mul_f32(galois_hip_ctx *ctx, const float *gate, const float *up, float *dst, int64_t k);
+/* cpy_f32_f32 / cpy_f32_f16, src/cuda.rs:1382-1595 -> cpy.cu:79-156 (also galois_cont): element i of the
+ * [ne00, ne01, *] source goes to element i of the [ne10, ne11, *] destination; nb* are BYTE strides as in
+ * the reference's F32Dim / F16Dim (src/cuda.rs:1360-1380). */
+int32_t galois_hip_cpy_f32(galois_hip_ctx *ctx, const void *x, void *dst, int32_t dst_is_f16, int64_t ne, int64_t ne00,
+                           int64_t ne01, int64_t nb00, int64_t nb01, int64_t nb02, int64_t ne10, int64_t ne11,
+                           int64_t nb10, int64_t nb11, int64_t nb12);
+/* get_rows for a Q4_0 table: GetRows::f_q_x_f32, src/op.rs:2546-2571 (CPU-only in the reference; its GPU
+ * arm is todo!(), src/op.rs:3281-3292): dst row i = to_f32(table row ids[i]), ncols % 32 == 0. */
+int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const int32_t *ids, float *dst,
+                                 int32_t ncols, int32_t nr);
+/* f32 x f32 batched matmul with galois's shape conventions; todo!() in the reference (src/cuda.rs:867-879,
+ * src/op.rs:1624-1662).  a = [K, N, ne02] with element strides a_s0, a_s1, a_s2 (one of a_s0, a_s1 must
+ * be 1, so permuted K/V-cache views work), b = [K, M, ne12] contiguous, dst = [N, M, ne12];
+ * a is broadcast over ne12 / ne02 like the quantized path (src/op.rs:1473-1483). */
+int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K, int32_t N,
+                               int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2);
+
 #ifdef __cplusplus
 }
 #endif

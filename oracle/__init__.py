@@ -58,6 +58,8 @@ def lib():
             "orc_soft_max_f32": (None, [f32p, f32p, i64, i64]),
             "orc_soft_max_causal_f32": (None, [f32p, f32p, i64, i64, i64, i64]),
             "orc_mul_mat_f32": (None, [f32p, f32p, f32p, i64, i64, i64, i64, i64, i64, i64, i64]),
+            "orc_cpy_f32": (None, [C.c_void_p, C.c_void_p, C.c_int] + [i64] * 11),
+            "orc_get_rows_q4_0": (None, [u8p, i32p, f32p, i64, i64]),
             "orc_sizeof_block_q4_0": (C.c_int, []),
             "orc_sizeof_block_q8_0": (C.c_int, []),
             "orc_have_avx2": (C.c_int, []),
@@ -232,4 +234,21 @@ def mul_mat_f32(a, b):
     out = np.empty((ne12, m, n), np.float32)
     lib().orc_mul_mat_f32(_p(a, C.c_float), _p(b, C.c_float), _p(out, C.c_float), k, n, m, ne02, ne12,
                           s0, s1, s2)
+    return out
+
+
+def cpy_f32(src, dst, ne, ne00, ne01, nb0, ne10, ne11, nb1):
+    """Strided copy (byte strides nb0 = (nb00, nb01, nb02), nb1 likewise) into a float32 or float16 array."""
+    assert src.dtype == np.float32 and dst.dtype in (np.float32, np.float16)
+    lib().orc_cpy_f32(src.ctypes.data_as(C.c_void_p), dst.ctypes.data_as(C.c_void_p), int(dst.dtype == np.float16),
+                      ne, ne00, ne01, nb0[0], nb0[1], nb0[2], ne10, ne11, nb1[0], nb1[1], nb1[2])
+    return dst
+
+
+def get_rows_q4_0(table, ids):
+    table = _u8(table)
+    ids = np.ascontiguousarray(ids, np.int32)
+    ncols = table.shape[1] // Q4_0_BYTES * QK
+    out = np.empty((ids.size, ncols), np.float32)
+    lib().orc_get_rows_q4_0(_p(table, C.c_uint8), _p(ids, C.c_int32), _p(out, C.c_float), ncols, ids.size)
     return out

@@ -27,7 +27,7 @@
  *   orc_rms_norm_f32 / orc_mul_f32 ..... closed form in numpy float64; constant-row case
  *   orc_rope_f32 ....................... closed form; pos=0 identity; norm preservation; additivity
  *   orc_soft_max_f32 ................... scipy.special.softmax in float64; row sums; -inf mask
- *   orc_add/scale/silu/cpy ............. numpy closed forms
+ *   orc_add/scale/silu/cpy/get_rows .... numpy closed forms (transpose / astype(float16) / row gather)
  */
 #include <math.h>
 #include <pthread.h>
@@ -470,4 +470,33 @@ void orc_mul_mat_f32(const float *a, const float *b, float *dst, int64_t K, int6
                 dst[(i2 * M + m) * N + n] = (float)acc;
             }
     }
+}
+
+/* cpy_f32_f32 / cpy_f32_f16, galois-kernels/src/cpy.cu:79-156: element i of the [ne00, ne01, *]
+ * source (byte strides nb00..nb02) goes to element i of the [ne10, ne11, *] destination
+ * (byte strides nb10..nb12); f16 destination rounds to nearest even. */
+void orc_cpy_f32(const void *cx, void *cdst, int dst_is_f16, int64_t ne, int64_t ne00, int64_t ne01, int64_t nb00,
+                 int64_t nb01, int64_t nb02, int64_t ne10, int64_t ne11, int64_t nb10, int64_t nb11, int64_t nb12) {
+    for (int64_t i = 0; i < ne; i++) {
+        const int64_t i02 = i / (ne00 * ne01), i01 = (i - i02 * ne01 * ne00) / ne00;
+        const int64_t i00 = i - i02 * ne01 * ne00 - i01 * ne00;
+        const int64_t i12 = i / (ne10 * ne11), i11 = (i - i12 * ne10 * ne11) / ne10;
+        const int64_t i10 = i - i12 * ne10 * ne11 - i11 * ne10;
+        float v;
+        memcpy(&v, (const char *)cx + i00 * nb00 + i01 * nb01 + i02 * nb02, 4);
+        char *d = (char *)cdst + i10 * nb10 + i11 * nb11 + i12 * nb12;
+        if (dst_is_f16) {
+            const uint16_t h = orc_f32_to_f16(v);
+            memcpy(d, &h, 2);
+        } else {
+            memcpy(d, &v, 4);
+        }
+    }
+}
+
+/* GetRows::f_q_x_f32, src/op.rs:2546-2571: dst row i = to_f32(table row ids[i]). */
+void orc_get_rows_q4_0(const void *table, const int32_t *ids, float *dst, int64_t ncols, int64_t nr) {
+    const int64_t row_bytes = ncols / QK4_0 * (int64_t)sizeof(orc_block_q4_0);
+    for (int64_t i = 0; i < nr; i++)
+        orc_dequantize_row_q4_0((const char *)table + ids[i] * row_bytes, dst + i * ncols, ncols);
 }

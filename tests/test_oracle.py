@@ -300,3 +300,19 @@ def test_soft_max():
         assert np.allclose(got[r, :last + 1], scipy.special.softmax(xc[r, :last + 1].astype(np.float64)),
                            rtol=1e-6)
     assert got[0, 0] == 1.0 and got[8, 0] == 1.0
+
+
+def test_cpy_and_get_rows():
+    rng = np.random.default_rng(14)
+    # permute [ne0=6, ne1=4, ne2=3] -> contiguous copy of the (ne1 <-> ne2)-swapped view, like galois_cont
+    x = rng.standard_normal((3, 4, 6)).astype(np.float32)          # numpy [ne2, ne1, ne0]
+    dst = np.zeros((4, 3, 6), np.float32)                           # want dst[i1, i2, i0] = x[i2, i1, i0]
+    # source viewed as [ne00=6, ne01=3, ne02=4] with strides of the swapped view
+    oracle.cpy_f32(x, dst, x.size, 6, 3, (4, 6 * 4 * 4, 6 * 4), 6, 3, (4, 6 * 4, 6 * 3 * 4))
+    assert np.array_equal(dst, x.transpose(1, 0, 2))
+    h = np.zeros((3, 4, 6), np.float16)
+    oracle.cpy_f32(x, h, x.size, 6, 4, (4, 24, 96), 6, 4, (2, 12, 48))
+    assert np.array_equal(h, x.astype(np.float16))
+    w = oracle.quantize_q4_0((rng.standard_normal((10, 64)) * 0.02).astype(np.float32))
+    ids = np.array([7, 0, 7, 9], np.int32)
+    assert np.array_equal(oracle.get_rows_q4_0(w, ids), npref.q4_0_dequant(w)[ids])
