@@ -142,6 +142,21 @@ class Device:
     def event_destroy(self, ev):
         self._check(self._lib.galois_hip_event_destroy(self._ctx, ev))
 
+    # -- stream capture ------------------------------------------------------------------
+    def graph_begin_capture(self):
+        self._check(self._lib.galois_hip_graph_begin_capture(self._ctx))
+
+    def graph_end_capture(self):
+        g = C.c_void_p()
+        self._check(self._lib.galois_hip_graph_end_capture(self._ctx, C.byref(g)))
+        return g
+
+    def graph_launch(self, graph):
+        self._check(self._lib.galois_hip_graph_launch(self._ctx, graph))
+
+    def graph_destroy(self, graph):
+        self._check(self._lib.galois_hip_graph_destroy(self._ctx, graph))
+
     # -- ops: same argument order as the C ABI ----------------------------------------
     def quantize_row_q4_0(self, x, y, k):
         self._check(self._lib.galois_hip_quantize_row_q4_0(self._ctx, _ptr(x), _ptr(y), k))

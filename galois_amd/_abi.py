@@ -32,6 +32,10 @@ PROTOTYPES = {
     "galois_hip_event_record": (i32, [c_ctx, c_ev]),
     "galois_hip_event_elapsed_ms": (i32, [c_ctx, c_ev, c_ev, C.POINTER(f32)]),
     "galois_hip_event_destroy": (i32, [c_ctx, c_ev]),
+    "galois_hip_graph_begin_capture": (i32, [c_ctx]),
+    "galois_hip_graph_end_capture": (i32, [c_ctx, C.POINTER(vp)]),
+    "galois_hip_graph_launch": (i32, [c_ctx, vp]),
+    "galois_hip_graph_destroy": (i32, [c_ctx, vp]),
     "galois_hip_quantize_row_q4_0": (i32, [c_ctx, vp, vp, C.c_int64]),
     "galois_hip_dequantize_row_q4_0": (i32, [c_ctx, vp, vp, C.c_int64]),
     "galois_hip_dequantize_mul_mat_vec_q4_0": (i32, [c_ctx, vp, vp, vp, i32, i32]),

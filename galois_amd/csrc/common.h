@@ -14,11 +14,21 @@ struct galois_hip_ctx {
     int32_t gemv_config;  // 0 = choose from the shape; GALOIS_HIP_GEMV_CONFIG=1..5 forces a kernel shape (tuning)
     void *ws;         // workspace owned by the context (fp16 activations of the prefill matmul)
     size_t ws_bytes;
+    void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul
+    bool capturing;   // between graph_begin_capture and graph_end_capture: nothing may allocate or block
     char last_error[256];
 };
 
+// galois_hip_ctx::scratch holds GH_PARTIAL_FLOATS floats of partial sums.
+constexpr int64_t GH_PARTIAL_FLOATS = 1 << 20;
+
 struct galois_hip_event {
     hipEvent_t ev;
+};
+
+struct galois_hip_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
 };
 
 // Q4_0 block exactly as the reference stores it (src/ggml_quants.rs:140-145).
@@ -48,6 +58,9 @@ static inline int32_t gh_hip(galois_hip_ctx *ctx, hipError_t e, const char *what
     do {                                               \
         if (!(cond)) return gh_fail((ctx), (status), (what)); \
     } while (0)
+
+// Calls that allocate, free or block are refused while the stream is being captured.
+#define GH_NOT_CAPTURING(ctx, what) GH_REQUIRE((ctx), !(ctx)->capturing, GALOIS_HIP_E_UNSUPPORTED, what " during a graph capture")
 
 // Binds the context's device to the calling thread, then checks the launch that follows.
 #define GH_BIND(ctx)                                                       \

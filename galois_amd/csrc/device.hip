@@ -38,10 +38,22 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     ctx->last_error[0] = 0;
     ctx->ws = nullptr;
     ctx->ws_bytes = 0;
+    ctx->scratch = nullptr;
+    ctx->capturing = false;
     const char *cfg = getenv("GALOIS_HIP_GEMV_CONFIG");
     ctx->gemv_config = cfg ? atoi(cfg) : 0;
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
+        delete ctx;
+        return (int32_t)e;
+    }
+    const size_t scratch_bytes = GH_PARTIAL_FLOATS * sizeof(float);
+    e = hipMalloc(&ctx->scratch, scratch_bytes);
+    if (e == hipSuccess) e = hipMemsetAsync(ctx->scratch, 0, scratch_bytes, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        if (ctx->scratch) (void)hipFree(ctx->scratch);
+        (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return (int32_t)e;
     }
@@ -54,6 +66,7 @@ int32_t galois_hip_destroy(galois_hip_ctx *ctx) {
     (void)hipSetDevice(ctx->ordinal);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
     hipError_t e = hipStreamDestroy(ctx->stream);
     delete ctx;
     return (int32_t)e;
@@ -85,6 +98,7 @@ int32_t galois_hip_device_info(galois_hip_ctx *ctx, char *name, int32_t name_cap
 
 int32_t galois_hip_alloc_zeros(galois_hip_ctx *ctx, size_t bytes, void **out) {
     GH_REQUIRE_CTX(ctx);
+    GH_NOT_CAPTURING(ctx, "alloc_zeros");
     GH_REQUIRE(ctx, out != nullptr, GALOIS_HIP_E_NULL, "alloc_zeros: out");
     *out = nullptr;
     GH_BIND(ctx);
@@ -103,6 +117,7 @@ int32_t galois_hip_alloc_zeros(galois_hip_ctx *ctx, size_t bytes, void **out) {
 
 int32_t galois_hip_free(galois_hip_ctx *ctx, void *dptr) {
     GH_REQUIRE_CTX(ctx);
+    GH_NOT_CAPTURING(ctx, "free");
     if (!dptr) return GALOIS_HIP_OK;
     GH_BIND(ctx);
     hipError_t e = hipStreamSynchronize(ctx->stream);
@@ -112,6 +127,7 @@ int32_t galois_hip_free(galois_hip_ctx *ctx, void *dptr) {
 
 int32_t galois_hip_htod_sync_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
     GH_REQUIRE_CTX(ctx);
+    GH_NOT_CAPTURING(ctx, "htod_sync_copy");
     if (bytes == 0) return GALOIS_HIP_OK;
     GH_REQUIRE(ctx, dst_dev && src_host, GALOIS_HIP_E_NULL, "htod_sync_copy");
     GH_BIND(ctx);
@@ -122,6 +138,7 @@ int32_t galois_hip_htod_sync_copy(galois_hip_ctx *ctx, void *dst_dev, const void
 
 int32_t galois_hip_dtoh_sync_copy(galois_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
     GH_REQUIRE_CTX(ctx);
+    GH_NOT_CAPTURING(ctx, "dtoh_sync_copy");
     if (bytes == 0) return GALOIS_HIP_OK;
     GH_REQUIRE(ctx, dst_host && src_dev, GALOIS_HIP_E_NULL, "dtoh_sync_copy");
     GH_BIND(ctx);
@@ -154,6 +171,7 @@ int32_t galois_hip_dtod_copy_2d(galois_hip_ctx *ctx, void *dst_dev, size_t dpitc
 
 int32_t galois_hip_synchronize(galois_hip_ctx *ctx) {
     GH_REQUIRE_CTX(ctx);
+    GH_NOT_CAPTURING(ctx, "synchronize");
     GH_BIND(ctx);
     return gh_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
 }
@@ -182,6 +200,7 @@ int32_t galois_hip_event_record(galois_hip_ctx *ctx, galois_hip_event *ev) {
 
 int32_t galois_hip_event_elapsed_ms(galois_hip_ctx *ctx, galois_hip_event *start, galois_hip_event *stop, float *ms) {
     GH_REQUIRE_CTX(ctx);
+    GH_NOT_CAPTURING(ctx, "event_elapsed_ms");
     GH_REQUIRE(ctx, start && stop && ms, GALOIS_HIP_E_NULL, "event_elapsed_ms");
     GH_BIND(ctx);
     hipError_t e = hipEventSynchronize(stop->ev);
@@ -196,6 +215,57 @@ int32_t galois_hip_event_destroy(galois_hip_ctx *ctx, galois_hip_event *ev) {
     hipError_t e = hipEventDestroy(ev->ev);
     delete ev;
     return gh_hip(ctx, e, "hipEventDestroy");
+}
+
+// ---- stream capture: a launch-bound op sequence recorded once and replayed as one HIP graph ----
+
+int32_t galois_hip_graph_begin_capture(galois_hip_ctx *ctx) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, !ctx->capturing, GALOIS_HIP_E_UNSUPPORTED, "graph_begin_capture: a capture is already open");
+    GH_BIND(ctx);
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e == hipSuccess) ctx->capturing = true;
+    return gh_hip(ctx, e, "hipStreamBeginCapture");
+}
+
+int32_t galois_hip_graph_end_capture(galois_hip_ctx *ctx, galois_hip_graph **out) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, out != nullptr, GALOIS_HIP_E_NULL, "graph_end_capture: out");
+    GH_REQUIRE(ctx, ctx->capturing, GALOIS_HIP_E_UNSUPPORTED, "graph_end_capture: no capture is open");
+    GH_BIND(ctx);
+    *out = nullptr;
+    ctx->capturing = false;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipStreamEndCapture");
+    hipGraphExec_t x = nullptr;
+    e = hipGraphInstantiate(&x, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return gh_hip(ctx, e, "hipGraphInstantiate");
+    }
+    galois_hip_graph *gr = new galois_hip_graph();
+    gr->graph = g, gr->exec = x;
+    *out = gr;
+    return GALOIS_HIP_OK;
+}
+
+int32_t galois_hip_graph_launch(galois_hip_ctx *ctx, galois_hip_graph *graph) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, graph != nullptr, GALOIS_HIP_E_NULL, "graph_launch");
+    GH_REQUIRE(ctx, !ctx->capturing, GALOIS_HIP_E_UNSUPPORTED, "graph_launch inside a capture");
+    GH_BIND(ctx);
+    return gh_hip(ctx, hipGraphLaunch(graph->exec, ctx->stream), "hipGraphLaunch");
+}
+
+int32_t galois_hip_graph_destroy(galois_hip_ctx *ctx, galois_hip_graph *graph) {
+    GH_REQUIRE_CTX(ctx);
+    if (!graph) return GALOIS_HIP_OK;
+    GH_BIND(ctx);
+    hipError_t e1 = hipGraphExecDestroy(graph->exec);
+    hipError_t e2 = hipGraphDestroy(graph->graph);
+    delete graph;
+    return gh_hip(ctx, e1 != hipSuccess ? e1 : e2, "hipGraphDestroy");
 }
 
 }  // extern "C"

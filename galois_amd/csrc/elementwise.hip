@@ -1,6 +1,5 @@
 // Elementwise, copy and gather kernels around the Q4_0 path (the reference's add / mul / scale /
-// silu / cpy kernels and the CPU-only get_rows), plus the f32 batched matmul the attention of a
-// decode step needs.  All are HBM-bound, one read and one write per element.
+// silu / cpy kernels and the CPU-only get_rows).  All are HBM-bound, one read and one write per element.
 #include "common.h"
 
 namespace {
@@ -86,66 +85,6 @@ __global__ __launch_bounds__(kEwThreads) void get_rows_q4_0(const uint16_t *__re
             out[b * 32 + 2 * j + 1] = (float)((int)((v >> 8) & 0xF) - 8) * d;
             out[b * 32 + 2 * j + 17] = (float)((int)((v >> 12) & 0xF) - 8) * d;
         }
-    }
-}
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_mov(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float wave_sum(float v) {
-    v += dpp_mov<0xB1>(v);
-    v += dpp_mov<0x4E>(v);
-    v += dpp_mov<0x141>(v);
-    v += dpp_mov<0x140>(v);
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
-    return v;
-}
-
-// f32 x f32 batched matmul, rows of `a` contiguous along K (a_s0 == 1): dst[i2][m][n] =
-// sum_k a[(i2/r2)*a_s2 + n*a_s1 + k] * b[(i2*M + m)*K + k].  One wave per (n, i2); the QK^T of
-// a decode step (K = head_dim, N = cached positions).
-__global__ __launch_bounds__(kEwThreads) void mul_mat_f32_krows(const float *__restrict__ a,
-                                                                const float *__restrict__ b, float *__restrict__ dst,
-                                                                int K, int N, int M, int r2, int64_t a_s1,
-                                                                int64_t a_s2) {
-    const int lane = threadIdx.x & 63;
-    const int n = blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
-    const int i2 = blockIdx.y;
-    if (n >= N) return;
-    const float *ar = a + (int64_t)(i2 / r2) * a_s2 + (int64_t)n * a_s1;
-    for (int m = 0; m < M; m++) {
-        const float *br = b + ((int64_t)i2 * M + m) * K;
-        float acc = 0.0f;
-        for (int k = lane; k < K; k += 64) acc = __builtin_fmaf(ar[k], br[k], acc);
-        acc = wave_sum(acc);
-        if (lane == 0) dst[((int64_t)i2 * M + m) * N + n] = acc;
-    }
-}
-
-// Same contraction when `a` is contiguous along N (a_s1 == 1, K strided by a_s0): the P.V of a
-// decode step (K = cached positions, N = head_dim).  A workgroup owns 64 columns n of one batch
-// slice; its 4 waves split K and combine through LDS.
-__global__ __launch_bounds__(kEwThreads) void mul_mat_f32_ncols(const float *__restrict__ a,
-                                                                const float *__restrict__ b, float *__restrict__ dst,
-                                                                int K, int N, int M, int r2, int64_t a_s0,
-                                                                int64_t a_s2) {
-    __shared__ float part[kEwThreads];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n = blockIdx.x * 64 + lane;
-    const int i2 = blockIdx.y;
-    const float *ab = a + (int64_t)(i2 / r2) * a_s2;
-    for (int m = 0; m < M; m++) {
-        const float *br = b + ((int64_t)i2 * M + m) * K;
-        float acc = 0.0f;
-        if (n < N)
-            for (int k = wave; k < K; k += kEwThreads / 64) acc = __builtin_fmaf(ab[(int64_t)k * a_s0 + n], br[k], acc);
-        part[threadIdx.x] = acc;
-        __syncthreads();
-        if (wave == 0 && n < N)
-            dst[((int64_t)i2 * M + m) * N + n] = (part[lane] + part[64 + lane]) + (part[128 + lane] + part[192 + lane]);
-        __syncthreads();
     }
 }
 
@@ -250,26 +189,6 @@ int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const i
     hipLaunchKernelGGL(get_rows_q4_0, dim3((nr + 3) / 4), dim3(kEwThreads), 0, ctx->stream, (const uint16_t *)table,
                        ids, dst, ncols / 32, nr);
     GH_LAUNCH_CHECK(ctx, "get_rows_q4_0 launch");
-}
-
-int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K, int32_t N,
-                               int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2) {
-    GH_REQUIRE_CTX(ctx);
-    GH_REQUIRE(ctx, a && b && dst, GALOIS_HIP_E_NULL, "mul_mat_f32");
-    GH_REQUIRE(ctx, K > 0 && N > 0 && M > 0 && ne02 > 0 && ne12 > 0 && ne12 % ne02 == 0 && ne12 <= 65535,
-               GALOIS_HIP_E_SHAPE, "mul_mat_f32");
-    GH_REQUIRE(ctx, a_s0 == 1 || a_s1 == 1, GALOIS_HIP_E_UNSUPPORTED,
-               "mul_mat_f32: a must be contiguous along K (a_s0 == 1) or along N (a_s1 == 1)");
-    GH_REQUIRE(ctx, gh_aligned(a, 4) && gh_aligned(b, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "mul_mat_f32");
-    GH_BIND(ctx);
-    const int r2 = ne12 / ne02;
-    if (a_s0 == 1)
-        hipLaunchKernelGGL(mul_mat_f32_krows, dim3((N + 3) / 4, ne12), dim3(kEwThreads), 0, ctx->stream, a, b, dst, K, N,
-                           M, r2, a_s1, a_s2);
-    else
-        hipLaunchKernelGGL(mul_mat_f32_ncols, dim3((N + 63) / 64, ne12), dim3(kEwThreads), 0, ctx->stream, a, b, dst, K,
-                           N, M, r2, a_s0, a_s2);
-    GH_LAUNCH_CHECK(ctx, "mul_mat_f32 launch");
 }
 
 }  // extern "C"

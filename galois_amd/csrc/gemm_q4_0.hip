@@ -446,6 +446,7 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
         // fp16 copy of X in the context's workspace (grown on demand, kept until the context dies)
         const size_t need = (size_t)M * K * sizeof(_Float16);
         if (ctx->ws_bytes < need) {
+            GH_NOT_CAPTURING(ctx, "mul_mat_q4_0_f32: growing the fp16 workspace");
             hipError_t e = hipStreamSynchronize(ctx->stream);
             if (e != hipSuccess) return gh_hip(ctx, e, "hipStreamSynchronize");
             if (ctx->ws) (void)hipFree(ctx->ws);

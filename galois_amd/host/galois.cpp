@@ -133,6 +133,36 @@ GResult Tensor::view(size_t elem_offset, size_t n_dims, const size_t *shape, Ten
     return ok();
 }
 
+GResult Tensor::view_strided(size_t elem_offset, size_t n_dims, const size_t *shape, const size_t *stride,
+                             Tensor *out) const {
+    if (n_dims == 0 || n_dims > 4) return err(GError::ShapeError, "rank must be 1..4");
+    if (blck_size(dtype_) != 1) return err(GError::Unimplemented, "strided views of quantized tensors");
+    Tensor t = *this;
+    t.dim_ = Dim();
+    t.dim_.n_dims = n_dims;
+    size_t last = 0;  // largest element offset the view reaches
+    for (size_t i = 0; i < 4; i++) {
+        t.dim_.shape[i] = i < n_dims ? shape[i] : 1;
+        t.dim_.stride[i] = i < n_dims ? stride[i] : (i ? t.dim_.stride[i - 1] * t.dim_.shape[i - 1] : 1);
+        if (t.dim_.shape[i] == 0) return err(GError::ShapeError, "view with an empty dimension");
+        last += (t.dim_.shape[i] - 1) * t.dim_.stride[i];
+    }
+    const size_t ts = type_size(dtype_);
+    if ((elem_offset + last + 1) * ts > avail_) return err(GError::ShapeError, "view exceeds the tensor");
+    t.avail_ = avail_ - elem_offset * ts;
+    t.ptr_ = (uint8_t *)ptr_ + elem_offset * ts;
+    *out = t;
+    return ok();
+}
+
+GResult Tensor::write(const void *bytes, size_t n) {
+    if (!dim_.ggml_is_contiguous(dtype_)) return err(GError::Unimplemented, "write into a strided view");
+    if (n != nbytes()) return err(GError::ShapeError, "write: byte count does not match the shape");
+    if (dev_.is_gpu()) return dev_.gpu->check(galois_hip_htod_sync_copy(dev_.gpu->ctx(), ptr_, bytes, n));
+    memcpy(ptr_, bytes, n);
+    return ok();
+}
+
 // ---- ops ----------------------------------------------------------------------------------------
 
 static bool all_gpu(std::initializer_list<const Tensor *> ts, std::shared_ptr<CudaDevice> *dev) {
@@ -144,13 +174,33 @@ static bool all_gpu(std::initializer_list<const Tensor *> ts, std::shared_ptr<Cu
     return true;
 }
 
+// f32 x f32 arm (the products over the KV cache).  The reference routes this case to a todo!()
+// (src/cuda.rs:994-1010) after a cuBLAS sgemm path for F16 weights (:698-782); here src0 may be
+// any strided 3-D view, so a permuted cache needs no cont() copy first.
+static GResult matmul_f32(const CudaDevice &dev, const Tensor &a, const Tensor &b, Tensor &dst) {
+    const Dim &ad = a.dim(), &bd = b.dim(), &dd = dst.dim();
+    if (ad.shape[0] != bd.shape[0]) return err(GError::ShapeError, "matmul: ne00 != ne10");
+    if (dd.shape[0] != ad.shape[1] || dd.shape[1] != bd.shape[1] || dd.shape[2] != bd.shape[2] || dd.shape[3] != bd.shape[3])
+        return err(GError::ShapeError, "matmul: dst shape must be [ne01, ne11, ne12, ne13]");
+    if (ad.shape[3] != 1 || bd.shape[3] != 1) return err(GError::Unimplemented, "matmul f32: 4-D batches");
+    if (ad.shape[2] == 0 || bd.shape[2] % ad.shape[2] != 0) return err(GError::ShapeError, "matmul: src0 must broadcast over ne12");
+    if (!bd.ggml_is_contiguous(b.dtype()) || !dd.ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "matmul f32: src1 and dst must be contiguous");
+    return dev.check(galois_hip_mul_mat_f32(dev.ctx(), (const float *)a.data(), (const float *)b.data(), (float *)dst.data(),
+                                            (int32_t)ad.shape[0], (int32_t)ad.shape[1], (int32_t)bd.shape[1],
+                                            (int32_t)ad.shape[2], (int32_t)bd.shape[2], (int64_t)ad.stride[0],
+                                            (int64_t)ad.stride[1], (int64_t)ad.stride[2]));
+}
+
 // galois_matmul, src/op.rs:3093-3111 -> CudaMatMul.map -> f_q_f32_f32 (src/cuda.rs:994-1139).
 GResult galois_matmul(const Tensor &a, const Tensor &b, Tensor &dst) {
     std::shared_ptr<CudaDevice> dev;
     if (!all_gpu({&a, &b, &dst}, &dev))
         return err(GError::Unimplemented, "galois_matmul: only (Gpu, Gpu, Gpu) operands on one device (the reference's other arms are todo!() or CPU)");
+    if (a.dtype() == GGmlType::F32 && b.dtype() == GGmlType::F32 && dst.dtype() == GGmlType::F32)
+        return matmul_f32(*dev, a, b, dst);
     if (!(a.dtype() == GGmlType::Q4_0 && b.dtype() == GGmlType::F32 && dst.dtype() == GGmlType::F32))
-        return err(GError::Unimplemented, "galois_matmul: only (Q4_0, F32) -> F32 (CudaMap2::map, src/cuda.rs:476-521)");
+        return err(GError::Unimplemented, "galois_matmul: only (Q4_0 | F32, F32) -> F32 (CudaMap2::map, src/cuda.rs:476-521)");
     const Dim &ad = a.dim(), &bd = b.dim(), &dd = dst.dim();
     const size_t ne00 = ad.shape[0], ne01 = ad.shape[1], ne02 = ad.shape[2], ne03 = ad.shape[3];
     const size_t ne10 = bd.shape[0], ne11 = bd.shape[1], ne12 = bd.shape[2], ne13 = bd.shape[3];
@@ -224,6 +274,90 @@ GResult galois_soft_max(const Tensor &src, Tensor &dst) {
         return err(GError::ShapeError, "soft_max: src and dst shapes differ");
     return dev->check(galois_hip_soft_max_f32(dev->ctx(), (const float *)src.data(), (float *)dst.data(),
                                               (int32_t)src.dim().shape[0], (int32_t)src.dim().nrows()));
+}
+
+// galois_add / galois_mul, src/op.rs:3073-3127 -> CudaAdd / CudaMul (src/cuda.rs:1190-1250):
+// kx = elements of src0, ky = ne10 * ne11 of src1, dst[i] = src0[i] op src1[i % ky].
+static GResult binary(const char *name, bool is_add, const Tensor &a, const Tensor &b, Tensor &dst) {
+    std::shared_ptr<CudaDevice> dev;
+    if (!all_gpu({&a, &b, &dst}, &dev)) return err(GError::Unimplemented, std::string(name) + ": only (Gpu, Gpu, Gpu)");
+    if (a.dtype() != GGmlType::F32 || b.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32)
+        return err(GError::Unimplemented, std::string(name) + ": F32 only");
+    if (!a.dim().ggml_is_contiguous(a.dtype()) || !b.dim().ggml_is_contiguous(b.dtype()) ||
+        !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, std::string(name) + ": contiguous operands only");
+    const int64_t kx = (int64_t)a.dim().elem_count(), ky = (int64_t)(b.dim().shape[0] * b.dim().shape[1]);
+    if ((int64_t)dst.dim().elem_count() != kx) return err(GError::ShapeError, std::string(name) + ": dst must have src0's element count");
+    auto fn = is_add ? galois_hip_add_f32 : galois_hip_mul_f32;
+    return dev->check(fn(dev->ctx(), (const float *)a.data(), (const float *)b.data(), (float *)dst.data(), kx, ky));
+}
+GResult galois_add(const Tensor &a, const Tensor &b, Tensor &dst) { return binary("galois_add", true, a, b, dst); }
+GResult galois_mul(const Tensor &a, const Tensor &b, Tensor &dst) { return binary("galois_mul", false, a, b, dst); }
+
+// galois_unary, src/op.rs:3232-3256 -> CudaSilu (src/cuda.rs:1665-1690).
+GResult galois_unary(const Tensor &src, Tensor &dst, UnaryOp op) {
+    std::shared_ptr<CudaDevice> dev;
+    if (!all_gpu({&src, &dst}, &dev)) return err(GError::Unimplemented, "galois_unary: only (Gpu, Gpu)");
+    if (op != UnaryOp::Silu) return err(GError::Unimplemented, "galois_unary: only Silu");
+    if (src.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32) return err(GError::Unimplemented, "galois_unary: F32 only");
+    if (src.dim().elem_count() != dst.dim().elem_count()) return err(GError::ShapeError, "unary: src and dst shapes differ");
+    if (!src.dim().ggml_is_contiguous(src.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_unary: contiguous operands only");
+    return dev->check(galois_hip_silu_f32(dev->ctx(), (const float *)src.data(), (float *)dst.data(),
+                                          (int64_t)src.dim().elem_count()));
+}
+
+// galois_scale, src/op.rs:3258-3279 -> CudaScale::f_g_c (src/cuda.rs:1621-1638): the factor is the first
+// element of src1.  The reference's (Gpu, Gpu, Gpu) arm would read device memory from the host; only the
+// (Gpu, Cpu, Gpu) arm is meaningful and kept.
+GResult galois_scale(const Tensor &src0, const Tensor &src1, Tensor &dst) {
+    std::shared_ptr<CudaDevice> dev;
+    if (!all_gpu({&src0, &dst}, &dev) || src1.device().is_gpu())
+        return err(GError::Unimplemented, "galois_scale: only (Gpu, Cpu, Gpu)");
+    if (src0.dtype() != GGmlType::F32 || src1.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32)
+        return err(GError::Unimplemented, "galois_scale: F32 only");
+    if (src1.dim().elem_count() == 0) return err(GError::ShapeError, "scale: empty factor tensor");
+    if (src0.dim().elem_count() != dst.dim().elem_count()) return err(GError::ShapeError, "scale: src and dst shapes differ");
+    if (!src0.dim().ggml_is_contiguous(src0.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_scale: contiguous operands only");
+    return dev->check(galois_hip_scale_f32(dev->ctx(), (const float *)src0.data(), (float *)dst.data(),
+                                           *(const float *)src1.data(), (int64_t)src0.dim().elem_count()));
+}
+
+// galois_cpy / galois_cont, src/op.rs:3171-3201 -> CudaCpy (src/cuda.rs:1382-1595): element i of the source
+// (in its own ne0/ne1/ne2 order and byte strides) goes to element i of the destination.
+GResult galois_cpy(const Tensor &src, Tensor &dst) {
+    std::shared_ptr<CudaDevice> dev;
+    if (!all_gpu({&src, &dst}, &dev)) return err(GError::Unimplemented, "galois_cpy: only (Gpu, Gpu)");
+    if (src.dtype() != GGmlType::F32 || (dst.dtype() != GGmlType::F32 && dst.dtype() != GGmlType::F16))
+        return err(GError::Unimplemented, "galois_cpy: F32 -> F32 | F16 only");
+    const Dim &sd = src.dim(), &dd = dst.dim();
+    if (sd.elem_count() != dd.elem_count()) return err(GError::ShapeError, "cpy: element counts differ");
+    if (sd.shape[3] != 1 || dd.shape[3] != 1) return err(GError::Unimplemented, "cpy: 4-D tensors (the kernel indexes three dims, cpy.cu:79-110)");
+    const int64_t ss = 4, ds = (int64_t)type_size(dst.dtype());
+    return dev->check(galois_hip_cpy_f32(dev->ctx(), src.data(), dst.data(), dst.dtype() == GGmlType::F16,
+                                         (int64_t)sd.elem_count(), (int64_t)sd.shape[0], (int64_t)sd.shape[1],
+                                         (int64_t)sd.stride[0] * ss, (int64_t)sd.stride[1] * ss, (int64_t)sd.stride[2] * ss,
+                                         (int64_t)dd.shape[0], (int64_t)dd.shape[1], (int64_t)dd.stride[0] * ds,
+                                         (int64_t)dd.stride[1] * ds, (int64_t)dd.stride[2] * ds));
+}
+GResult galois_cont(const Tensor &src, Tensor &dst) {
+    if (!dst.dim().ggml_is_contiguous(dst.dtype())) return err(GError::ShapeError, "cont: dst must be contiguous");
+    return galois_cpy(src, dst);
+}
+
+// galois_get_rows, src/op.rs:3281-3292 -> GetRows::f_q_x_f32 (src/op.rs:2546-2571), on the device.
+GResult galois_get_rows(const Tensor &src0, const Tensor &src1, Tensor &dst) {
+    std::shared_ptr<CudaDevice> dev;
+    if (!all_gpu({&src0, &src1, &dst}, &dev)) return err(GError::Unimplemented, "galois_get_rows: only (Gpu, Gpu, Gpu)");
+    if (src0.dtype() != GGmlType::Q4_0 || src1.dtype() != GGmlType::I32 || dst.dtype() != GGmlType::F32)
+        return err(GError::Unimplemented, "galois_get_rows: (Q4_0, I32) -> F32 only");
+    const size_t nc = src0.dim().shape[0], nr = src1.dim().elem_count();
+    if (dst.dim().shape[0] != nc || dst.dim().elem_count() != nc * nr) return err(GError::ShapeError, "get_rows: dst must be [ne00, n_ids]");
+    if (!src0.dim().ggml_is_contiguous(src0.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_get_rows: contiguous operands only");
+    return dev->check(galois_hip_get_rows_q4_0(dev->ctx(), src0.data(), (const int32_t *)src1.data(), (float *)dst.data(),
+                                               (int32_t)nc, (int32_t)nr));
 }
 
 }  // namespace galois

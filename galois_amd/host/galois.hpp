@@ -70,6 +70,10 @@ class Tensor {
     GResult to_cpu_tensor(Tensor *out) const;
     // view with another shape over the same storage (view_tensor): offset in storage elements
     GResult view(size_t elem_offset, size_t n_dims, const size_t *shape, Tensor *out) const;
+    // view with explicit strides in storage elements (what permute / transpose produce in the reference)
+    GResult view_strided(size_t elem_offset, size_t n_dims, const size_t *shape, const size_t *stride, Tensor *out) const;
+    // overwrite the tensor's bytes from host memory (synchronous)
+    GResult write(const void *bytes, size_t nbytes);
 
     GGmlType dtype() const { return dtype_; }
     const Dim &dim() const { return dim_; }
@@ -103,5 +107,14 @@ GResult galois_matmul(const Tensor &a, const Tensor &b, Tensor &dst);           
 GResult galois_rms_norm(const Tensor &src, Tensor &dst, float eps);                                      // op.rs:3155-3169
 GResult galois_rope_custom(const RopeCustomOption &op, const Tensor &src0, const Tensor &src1, Tensor &dst);  // op.rs:3304-3341
 GResult galois_soft_max(const Tensor &src, Tensor &dst);                                                  // op.rs:3216-3230
+
+enum class UnaryOp { Silu };  // the only arm the reference implements, src/op.rs:3232-3256
+GResult galois_add(const Tensor &a, const Tensor &b, Tensor &dst);          // op.rs:3073-3091
+GResult galois_mul(const Tensor &a, const Tensor &b, Tensor &dst);          // op.rs:3113-3127
+GResult galois_unary(const Tensor &src, Tensor &dst, UnaryOp op);           // op.rs:3232-3256
+GResult galois_scale(const Tensor &src0, const Tensor &src1, Tensor &dst);  // op.rs:3258-3279 (src1: one f32, Cpu or Gpu)
+GResult galois_cpy(const Tensor &src, Tensor &dst);                         // op.rs:3171-3185
+GResult galois_cont(const Tensor &src, Tensor &dst);                        // op.rs:3187-3201
+GResult galois_get_rows(const Tensor &src0, const Tensor &src1, Tensor &dst);  // op.rs:3281-3292 (Gpu arm is todo!() there)
 
 }  // namespace galois

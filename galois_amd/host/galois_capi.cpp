@@ -3,6 +3,7 @@
 #include <string>
 
 #include "galois.hpp"
+#include "llama.hpp"
 
 using namespace galois;
 
@@ -89,6 +90,119 @@ int galois_host_rope_custom(size_t n_dims, int mode, int n_ctx, float freq_base,
 int galois_host_soft_max(void *src, void *dst) {
     GResult r = galois_soft_max(*(Tensor *)src, *(Tensor *)dst);
     return r.ok() ? 0 : fail(r);
+}
+
+void *galois_host_tensor_view_strided(void *src, size_t elem_offset, size_t n_dims, const size_t *shape, const size_t *stride) {
+    auto *t = new Tensor();
+    GResult r = ((Tensor *)src)->view_strided(elem_offset, n_dims, shape, stride, t);
+    if (!r.ok()) {
+        fail(r);
+        delete t;
+        return nullptr;
+    }
+    return t;
+}
+int galois_host_tensor_write(void *t, const void *bytes, size_t nbytes) {
+    GResult r = ((Tensor *)t)->write(bytes, nbytes);
+    return r.ok() ? 0 : fail(r);
+}
+void *galois_host_tensor_data(void *t) { return ((Tensor *)t)->data(); }
+
+int galois_host_add(void *a, void *b, void *dst) {
+    GResult r = galois_add(*(Tensor *)a, *(Tensor *)b, *(Tensor *)dst);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_mul(void *a, void *b, void *dst) {
+    GResult r = galois_mul(*(Tensor *)a, *(Tensor *)b, *(Tensor *)dst);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_unary_silu(void *src, void *dst) {
+    GResult r = galois_unary(*(Tensor *)src, *(Tensor *)dst, UnaryOp::Silu);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_scale(void *src0, void *src1, void *dst) {
+    GResult r = galois_scale(*(Tensor *)src0, *(Tensor *)src1, *(Tensor *)dst);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_cpy(void *src, void *dst) {
+    GResult r = galois_cpy(*(Tensor *)src, *(Tensor *)dst);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_cont(void *src, void *dst) {
+    GResult r = galois_cont(*(Tensor *)src, *(Tensor *)dst);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_get_rows(void *src0, void *src1, void *dst) {
+    GResult r = galois_get_rows(*(Tensor *)src0, *(Tensor *)src1, *(Tensor *)dst);
+    return r.ok() ? 0 : fail(r);
+}
+
+// ---- LLaMA decode driver -------------------------------------------------------------------------
+void *galois_host_llama_new(void *dev, size_t n_vocab, size_t n_embd, size_t n_head, size_t n_layer, size_t n_ff,
+                            size_t n_ctx, float rms_eps, float freq_base) {
+    LlamaHParams hp;
+    hp.n_vocab = n_vocab, hp.n_embd = n_embd, hp.n_head = n_head, hp.n_layer = n_layer, hp.n_ff = n_ff, hp.n_ctx = n_ctx;
+    hp.rms_eps = rms_eps, hp.freq_base = freq_base;
+    std::unique_ptr<LlamaDecoder> m;
+    GResult r = LlamaDecoder::create(hp, *(Device *)dev, &m);
+    if (!r.ok()) {
+        fail(r);
+        return nullptr;
+    }
+    return m.release();
+}
+void galois_host_llama_free(void *m) { delete (LlamaDecoder *)m; }
+// borrowed handle: valid while the decoder lives, never passed to galois_host_tensor_free
+void *galois_host_llama_tensor(void *m, const char *name, int layer) {
+    Tensor *t = ((LlamaDecoder *)m)->tensor(name, layer);
+    if (!t) fail(GError{GError::Unexpected, std::string("no tensor named ") + name});
+    return t;
+}
+void *galois_host_llama_logits(void *m) { return (void *)&((LlamaDecoder *)m)->logits(); }
+size_t galois_host_llama_ops_per_step(void *m) { return ((LlamaDecoder *)m)->ops_per_step(); }
+int galois_host_llama_decode(void *m, int32_t token, int32_t n_past, int fused) {
+    GResult r = ((LlamaDecoder *)m)->decode(token, n_past, fused != 0);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_llama_capture(void *m, int32_t token, int32_t n_past, int fused) {
+    GResult r = ((LlamaDecoder *)m)->capture(token, n_past, fused != 0);
+    return r.ok() ? 0 : fail(r);
+}
+int galois_host_llama_replay(void *m) {
+    GResult r = ((LlamaDecoder *)m)->replay();
+    return r.ok() ? 0 : fail(r);
+}
+// replays the captured step `n` times between two events; milliseconds for all n in *ms
+int galois_host_llama_time_replays(void *m, void *dev, int n, float *ms) {
+    galois_hip_ctx *ctx = ((Device *)dev)->gpu->ctx();
+    galois_hip_event *e0 = nullptr, *e1 = nullptr;
+    int32_t st = galois_hip_event_create(ctx, &e0);
+    if (!st) st = galois_hip_event_create(ctx, &e1);
+    if (!st) st = galois_hip_event_record(ctx, e0);
+    GResult r;
+    for (int i = 0; i < n && !st && r.ok(); i++) r = ((LlamaDecoder *)m)->replay();
+    if (!st) st = galois_hip_event_record(ctx, e1);
+    if (!st) st = galois_hip_event_elapsed_ms(ctx, e0, e1, ms);
+    galois_hip_event_destroy(ctx, e0);
+    galois_hip_event_destroy(ctx, e1);
+    if (!r.ok()) return fail(r);
+    return st ? fail(GError{GError::DeviceError, galois_hip_last_error(ctx)}) : 0;
+}
+// same for eager steps (op-by-op launches)
+int galois_host_llama_time_steps(void *m, void *dev, int32_t token, int32_t n_past, int fused, int n, float *ms) {
+    galois_hip_ctx *ctx = ((Device *)dev)->gpu->ctx();
+    galois_hip_event *e0 = nullptr, *e1 = nullptr;
+    int32_t st = galois_hip_event_create(ctx, &e0);
+    if (!st) st = galois_hip_event_create(ctx, &e1);
+    if (!st) st = galois_hip_event_record(ctx, e0);
+    GResult r;
+    for (int i = 0; i < n && !st && r.ok(); i++) r = ((LlamaDecoder *)m)->decode(token, n_past, fused != 0);
+    if (!st) st = galois_hip_event_record(ctx, e1);
+    if (!st) st = galois_hip_event_elapsed_ms(ctx, e0, e1, ms);
+    galois_hip_event_destroy(ctx, e0);
+    galois_hip_event_destroy(ctx, e1);
+    if (!r.ok()) return fail(r);
+    return st ? fail(GError{GError::DeviceError, galois_hip_last_error(ctx)}) : 0;
 }
 
 }  // extern "C"

@@ -1,0 +1,227 @@
+// LLaMA decode step over the galois op mirror (see llama.hpp).
+#include "llama.hpp"
+
+#include <cmath>
+
+namespace galois {
+
+static GError err(GError::Kind k, const std::string &m) { return GError{k, m}; }
+
+#define G_TRY(expr)              \
+    do {                         \
+        GResult r__ = (expr);    \
+        if (!r__.ok()) return r__; \
+    } while (0)
+
+GResult galois_rms_norm_mul(const Tensor &src, const Tensor &weight, Tensor &dst, float eps) {
+    if (!src.device().is_gpu() || !weight.device().is_gpu() || !dst.device().is_gpu())
+        return err(GError::Unimplemented, "galois_rms_norm_mul: only (Gpu, Gpu, Gpu)");
+    if (src.dtype() != GGmlType::F32 || weight.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32)
+        return err(GError::Unimplemented, "galois_rms_norm_mul: F32 only");
+    if (weight.dim().elem_count() != src.dim().shape[0] || src.dim().elem_count() != dst.dim().elem_count())
+        return err(GError::ShapeError, "rms_norm_mul: weight must have ne00 elements, dst the shape of src");
+    const auto &dev = src.device().gpu;
+    return dev->check(galois_hip_rms_norm_mul_f32(dev->ctx(), (const float *)src.data(), (const float *)weight.data(),
+                                                  (float *)dst.data(), (int32_t)src.dim().shape[0],
+                                                  (int32_t)src.dim().nrows(), eps));
+}
+
+GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst) {
+    if (!gate.device().is_gpu() || !up.device().is_gpu() || !dst.device().is_gpu())
+        return err(GError::Unimplemented, "galois_silu_mul: only (Gpu, Gpu, Gpu)");
+    if (gate.dtype() != GGmlType::F32 || up.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32)
+        return err(GError::Unimplemented, "galois_silu_mul: F32 only");
+    if (gate.dim().elem_count() != up.dim().elem_count() || gate.dim().elem_count() != dst.dim().elem_count())
+        return err(GError::ShapeError, "silu_mul: shapes differ");
+    const auto &dev = gate.device().gpu;
+    return dev->check(galois_hip_silu_mul_f32(dev->ctx(), (const float *)gate.data(), (const float *)up.data(),
+                                              (float *)dst.data(), (int64_t)gate.dim().elem_count()));
+}
+
+static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t ne1 = 0, size_t ne2 = 0) {
+    const size_t shape[3] = {ne0, ne1, ne2};
+    return Tensor::zeros(ne2 ? 3 : (ne1 ? 2 : 1), shape, ty, dev, t);
+}
+
+GResult LlamaDecoder::create(const LlamaHParams &hp, const Device &dev, std::unique_ptr<LlamaDecoder> *out) {
+    if (!dev.is_gpu()) return err(GError::Unimplemented, "LlamaDecoder: Gpu device only");
+    if (hp.n_head == 0 || hp.n_embd % hp.n_head != 0 || (hp.n_embd / hp.n_head) % 2 != 0)
+        return err(GError::ShapeError, "LlamaDecoder: n_embd must split into n_head even-sized heads");
+    if (hp.n_embd % 32 != 0 || hp.n_ff % 32 != 0) return err(GError::ShapeError, "LlamaDecoder: n_embd and n_ff must be multiples of 32");
+    std::unique_ptr<LlamaDecoder> m(new LlamaDecoder());
+    m->hp_ = hp;
+    m->dev_ = dev;
+    const size_t E = hp.n_embd, F = hp.n_ff, V = hp.n_vocab, C = hp.n_ctx, H = hp.n_head, D = E / H;
+    const GGmlType Q = GGmlType::Q4_0, F32 = GGmlType::F32;
+    G_TRY(mk(&m->tok_embd_, Q, dev, E, V));
+    G_TRY(mk(&m->out_norm_, F32, dev, E));
+    G_TRY(mk(&m->output_, Q, dev, E, V));
+    m->layers_.resize(hp.n_layer);
+    for (Layer &l : m->layers_) {
+        G_TRY(mk(&l.attn_norm, F32, dev, E));
+        G_TRY(mk(&l.ffn_norm, F32, dev, E));
+        G_TRY(mk(&l.wq, Q, dev, E, E));
+        G_TRY(mk(&l.wk, Q, dev, E, E));
+        G_TRY(mk(&l.wv, Q, dev, E, E));
+        G_TRY(mk(&l.wo, Q, dev, E, E));
+        G_TRY(mk(&l.w_gate, Q, dev, E, F));
+        G_TRY(mk(&l.w_up, Q, dev, E, F));
+        G_TRY(mk(&l.w_down, Q, dev, F, E));
+        G_TRY(mk(&l.k_cache, F32, dev, E, C));
+        G_TRY(mk(&l.v_cache, F32, dev, E, C));
+    }
+    G_TRY(mk(&m->tok_id_, GGmlType::I32, dev, 1));
+    G_TRY(mk(&m->pos_, GGmlType::I32, dev, 1));
+    G_TRY(mk(&m->scale_, F32, Device{}, 1));
+    *(float *)m->scale_.data() = 1.0f / sqrtf((float)D);
+    for (Tensor *t : {&m->x_, &m->t_, &m->a_, &m->q_, &m->k_, &m->v_, &m->ao_, &m->x1_, &m->f_, &m->d_}) G_TRY(mk(t, F32, dev, E, 1));
+    G_TRY(mk(&m->qr_, F32, dev, D, H, 1));
+    G_TRY(mk(&m->kr_, F32, dev, D, H, 1));
+    G_TRY(mk(&m->s_, F32, dev, C, 1, H));
+    G_TRY(mk(&m->p_, F32, dev, C, 1, H));
+    G_TRY(mk(&m->o_, F32, dev, D, 1, H));
+    for (Tensor *t : {&m->g_, &m->u_, &m->h_}) G_TRY(mk(t, F32, dev, F, 1));
+    G_TRY(mk(&m->logits_, F32, dev, V, 1));
+    *out = std::move(m);
+    return GError{};
+}
+
+LlamaDecoder::~LlamaDecoder() {
+    if (graph_) galois_hip_graph_destroy(dev_.gpu->ctx(), graph_);
+}
+
+Tensor *LlamaDecoder::tensor(const std::string &name, int layer) {
+    if (layer < 0) {
+        if (name == "tok_embd") return &tok_embd_;
+        if (name == "out_norm") return &out_norm_;
+        if (name == "output") return &output_;
+        return nullptr;
+    }
+    if ((size_t)layer >= layers_.size()) return nullptr;
+    Layer &l = layers_[layer];
+    const std::pair<const char *, Tensor *> names[] = {
+        {"attn_norm", &l.attn_norm}, {"ffn_norm", &l.ffn_norm}, {"wq", &l.wq}, {"wk", &l.wk}, {"wv", &l.wv}, {"wo", &l.wo},
+        {"w_gate", &l.w_gate}, {"w_up", &l.w_up}, {"w_down", &l.w_down}, {"k_cache", &l.k_cache}, {"v_cache", &l.v_cache}};
+    for (const auto &n : names)
+        if (name == n.first) return n.second;
+    return nullptr;
+}
+
+GResult LlamaDecoder::set_inputs(int32_t token, int32_t n_past) {
+    if (token < 0 || (size_t)token >= hp_.n_vocab) return err(GError::ShapeError, "decode: token id out of range");
+    if (n_past < 0 || (size_t)n_past >= hp_.n_ctx) return err(GError::ShapeError, "decode: n_past must be below n_ctx");
+    if (token != last_token_) G_TRY(tok_id_.write(&token, sizeof(token)));  // synchronous copies: only when they change
+    if (n_past != last_pos_) G_TRY(pos_.write(&n_past, sizeof(n_past)));
+    last_token_ = token, last_pos_ = n_past;
+    return GError{};
+}
+
+// The op sequence of one token.  Shapes in ggml order [ne0, ne1, ne2]; L = n_past + 1 keys are visible,
+// so the softmax needs no mask.
+GResult LlamaDecoder::step(int32_t n_past, bool fused) {
+    const size_t E = hp_.n_embd, H = hp_.n_head, D = E / H, L = (size_t)n_past + 1, C = hp_.n_ctx;
+    RopeCustomOption rope;
+    rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;
+    size_t ops = 0;
+    auto norm = [&](const Tensor &src, const Tensor &w, Tensor &dst) -> GResult {
+        if (fused) {
+            ops += 1;
+            return galois_rms_norm_mul(src, w, dst, hp_.rms_eps);
+        }
+        ops += 2;
+        G_TRY(galois_rms_norm(src, t_, hp_.rms_eps));
+        return galois_mul(t_, w, dst);
+    };
+    // views that depend on L: the first L scores of every head are packed as [L, 1, H]
+    Tensor s, p, q3, k_row, v_row;
+    {
+        const size_t sh[3] = {L, 1, H};
+        G_TRY(s_.view(0, 3, sh, &s));
+        G_TRY(p_.view(0, 3, sh, &p));
+        const size_t qs[3] = {D, 1, H};
+        G_TRY(qr_.view(0, 3, qs, &q3));
+    }
+    G_TRY(galois_get_rows(tok_embd_, tok_id_, x_)); ops++;
+    for (Layer &l : layers_) {
+        G_TRY(norm(x_, l.attn_norm, a_));
+        G_TRY(galois_matmul(l.wq, a_, q_));
+        G_TRY(galois_matmul(l.wk, a_, k_));
+        G_TRY(galois_matmul(l.wv, a_, v_)); ops += 3;
+        Tensor qv, kv;
+        const size_t hs[3] = {D, H, 1};
+        G_TRY(q_.view(0, 3, hs, &qv));
+        G_TRY(k_.view(0, 3, hs, &kv));
+        G_TRY(galois_rope_custom(rope, qv, pos_, qr_));
+        G_TRY(galois_rope_custom(rope, kv, pos_, kr_)); ops += 2;
+        // append this position to the cache
+        const size_t row[2] = {E, 1};
+        G_TRY(l.k_cache.view((size_t)n_past * E, 2, row, &k_row));
+        G_TRY(l.v_cache.view((size_t)n_past * E, 2, row, &v_row));
+        Tensor kr_flat;
+        G_TRY(kr_.view(0, 2, row, &kr_flat));
+        G_TRY(galois_cpy(kr_flat, k_row));
+        G_TRY(galois_cpy(v_, v_row)); ops += 2;
+        // scores = K^T q per head: K seen as [D, L, H] with strides (1, E, D)
+        Tensor kc, vc;
+        const size_t ksh[3] = {D, L, H}, kst[3] = {1, E, D};
+        G_TRY(l.k_cache.view_strided(0, 3, ksh, kst, &kc));
+        G_TRY(galois_matmul(kc, q3, s));
+        G_TRY(galois_scale(s, scale_, s));
+        G_TRY(galois_soft_max(s, p)); ops += 3;
+        // out = V p per head: V seen as [L, D, H] with strides (E, 1, D)
+        const size_t vsh[3] = {L, D, H}, vst[3] = {E, 1, D};
+        G_TRY(l.v_cache.view_strided(0, 3, vsh, vst, &vc));
+        G_TRY(galois_matmul(vc, p, o_)); ops++;
+        Tensor o_flat;
+        G_TRY(o_.view(0, 2, row, &o_flat));
+        G_TRY(galois_matmul(l.wo, o_flat, ao_));
+        G_TRY(galois_add(ao_, x_, x1_)); ops += 2;
+        G_TRY(norm(x1_, l.ffn_norm, f_));
+        G_TRY(galois_matmul(l.w_gate, f_, g_));
+        G_TRY(galois_matmul(l.w_up, f_, u_)); ops += 2;
+        if (fused) {
+            G_TRY(galois_silu_mul(g_, u_, h_)); ops++;
+        } else {
+            G_TRY(galois_unary(g_, h_, UnaryOp::Silu));
+            G_TRY(galois_mul(h_, u_, h_)); ops += 2;
+        }
+        G_TRY(galois_matmul(l.w_down, h_, d_));
+        G_TRY(galois_add(d_, x1_, x_)); ops += 2;
+    }
+    G_TRY(norm(x_, out_norm_, a_));
+    G_TRY(galois_matmul(output_, a_, logits_)); ops++;
+    n_ops_ = ops;
+    return GError{};
+}
+
+GResult LlamaDecoder::decode(int32_t token, int32_t n_past, bool fused) {
+    G_TRY(set_inputs(token, n_past));
+    return step(n_past, fused);
+}
+
+GResult LlamaDecoder::capture(int32_t token, int32_t n_past, bool fused) {
+    galois_hip_ctx *ctx = dev_.gpu->ctx();
+    if (graph_) {
+        G_TRY(dev_.gpu->check(galois_hip_graph_destroy(ctx, graph_)));
+        graph_ = nullptr;
+    }
+    G_TRY(set_inputs(token, n_past));
+    G_TRY(dev_.gpu->check(galois_hip_graph_begin_capture(ctx)));
+    GResult r = step(n_past, fused);
+    galois_hip_graph *g = nullptr;
+    GResult e = dev_.gpu->check(galois_hip_graph_end_capture(ctx, &g));  // always close the capture
+    if (!r.ok()) {
+        if (g) galois_hip_graph_destroy(ctx, g);
+        return r;
+    }
+    G_TRY(e);
+    graph_ = g;
+    return GError{};
+}
+
+GResult LlamaDecoder::replay() {
+    if (!graph_) return err(GError::Unexpected, "replay: no step has been captured");
+    return dev_.gpu->check(galois_hip_graph_launch(dev_.gpu->ctx(), graph_));
+}
+
+}  // namespace galois

@@ -1,0 +1,68 @@
+// One-token decode step of a LLaMA-architecture model written with the galois ops of galois.hpp.
+//
+// The reference ships no model graph (its consumer is external, example/src/main.rs:4); the op set it
+// registers (src/kernels.rs:5-20) is the ggml-era LLaMA graph, and this driver issues exactly that
+// sequence: get_rows, rms_norm, mul, matmul (Q4_0 and f32), rope_custom, cpy, scale, soft_max, unary
+// (Silu) and add.  Linear weights are Q4_0, norms and the KV cache f32.  The step can be issued op by
+// op or recorded once and replayed as a HIP graph.
+#pragma once
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "galois.hpp"
+
+namespace galois {
+
+struct LlamaHParams {
+    size_t n_vocab = 32000, n_embd = 4096, n_head = 32, n_layer = 32, n_ff = 11008, n_ctx = 2048;
+    float rms_eps = 1e-6f, freq_base = 10000.0f, freq_scale = 1.0f;
+};
+
+class LlamaDecoder {
+   public:
+    // Allocates zeroed weights, the KV cache ([n_embd, n_ctx] f32 per layer, for K and for V) and every
+    // intermediate of a step, so that decode() itself allocates nothing.
+    static GResult create(const LlamaHParams &hp, const Device &dev, std::unique_ptr<LlamaDecoder> *out);
+    ~LlamaDecoder();
+
+    // Weights by name: "tok_embd" [n_embd, n_vocab] Q4_0, "out_norm" [n_embd] F32, "output" [n_embd, n_vocab] Q4_0
+    // (layer = -1), and per layer "attn_norm", "ffn_norm" F32, "wq", "wk", "wv", "wo" [n_embd, n_embd],
+    // "w_gate", "w_up" [n_embd, n_ff], "w_down" [n_ff, n_embd] Q4_0, "k_cache", "v_cache" [n_embd, n_ctx] F32.
+    Tensor *tensor(const std::string &name, int layer);
+
+    // Enqueues one step for `token` at position n_past (attention over n_past + 1 keys); logits() holds the
+    // result once the stream is synchronised (to_cpu_tensor does that).  fused = use the library's fused
+    // rms_norm*weight and silu*up kernels instead of two ops each.
+    GResult decode(int32_t token, int32_t n_past, bool fused);
+    // Records the same step as a graph / replays the recorded step.
+    GResult capture(int32_t token, int32_t n_past, bool fused);
+    GResult replay();
+    const Tensor &logits() const { return logits_; }
+    const LlamaHParams &hparams() const { return hp_; }
+    size_t ops_per_step() const { return n_ops_; }
+
+   private:
+    struct Layer {
+        Tensor attn_norm, ffn_norm, wq, wk, wv, wo, w_gate, w_up, w_down, k_cache, v_cache;
+    };
+    GResult set_inputs(int32_t token, int32_t n_past);
+    GResult step(int32_t n_past, bool fused);
+
+    LlamaHParams hp_;
+    Device dev_;
+    Tensor tok_embd_, out_norm_, output_;
+    std::vector<Layer> layers_;
+    Tensor tok_id_, pos_, scale_;                                    // I32 [1], I32 [1], host f32 [1]
+    Tensor x_, t_, a_, q_, k_, v_, qr_, kr_, s_, p_, o_, ao_, x1_, f_, g_, u_, h_, d_, logits_;
+    galois_hip_graph *graph_ = nullptr;
+    size_t n_ops_ = 0;
+    int32_t last_token_ = -1, last_pos_ = -1;
+};
+
+// Extensions used by the fused mode (no counterpart in the reference's op list): rms_norm followed by the
+// weight multiply, and silu(gate) * up, each as one kernel.
+GResult galois_rms_norm_mul(const Tensor &src, const Tensor &weight, Tensor &dst, float eps);
+GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst);
+
+}  // namespace galois

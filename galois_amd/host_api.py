@@ -45,7 +45,22 @@ def lib():
                 ("galois_host_rms_norm", C.c_int, [vp, vp, C.c_float]),
                 ("galois_host_rope_custom", C.c_int, [sz, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int,
                                                       vp, vp, vp]),
-                ("galois_host_soft_max", C.c_int, [vp, vp])):
+                ("galois_host_soft_max", C.c_int, [vp, vp]),
+                ("galois_host_tensor_view_strided", vp, [vp, sz, sz, C.POINTER(sz), C.POINTER(sz)]),
+                ("galois_host_tensor_write", C.c_int, [vp, vp, sz]), ("galois_host_tensor_data", vp, [vp]),
+                ("galois_host_add", C.c_int, [vp, vp, vp]), ("galois_host_mul", C.c_int, [vp, vp, vp]),
+                ("galois_host_unary_silu", C.c_int, [vp, vp]), ("galois_host_scale", C.c_int, [vp, vp, vp]),
+                ("galois_host_cpy", C.c_int, [vp, vp]), ("galois_host_cont", C.c_int, [vp, vp]),
+                ("galois_host_get_rows", C.c_int, [vp, vp, vp]),
+                ("galois_host_llama_new", vp, [vp, sz, sz, sz, sz, sz, sz, C.c_float, C.c_float]),
+                ("galois_host_llama_free", None, [vp]), ("galois_host_llama_tensor", vp, [vp, C.c_char_p, C.c_int]),
+                ("galois_host_llama_logits", vp, [vp]), ("galois_host_llama_ops_per_step", sz, [vp]),
+                ("galois_host_llama_decode", C.c_int, [vp, C.c_int32, C.c_int32, C.c_int]),
+                ("galois_host_llama_capture", C.c_int, [vp, C.c_int32, C.c_int32, C.c_int]),
+                ("galois_host_llama_replay", C.c_int, [vp]),
+                ("galois_host_llama_time_replays", C.c_int, [vp, vp, C.c_int, C.POINTER(C.c_float)]),
+                ("galois_host_llama_time_steps", C.c_int, [vp, vp, C.c_int32, C.c_int32, C.c_int, C.c_int,
+                                                           C.POINTER(C.c_float)])):
             fn = getattr(L, name)
             fn.restype, fn.argtypes = res, args
         _lib = L
@@ -107,6 +122,22 @@ class Tensor:
             _raise(2)
         return Tensor(h, shape, self.dtype)
 
+    def view_strided(self, elem_offset, shape, stride):
+        """A view with explicit strides in elements (what permute / transpose give in the reference)."""
+        n, sh = _shape(shape)
+        _, st = _shape(stride)
+        h = lib().galois_host_tensor_view_strided(self.h, elem_offset, n, sh, st)
+        if not h:
+            _raise(2)
+        return Tensor(h, shape, self.dtype)
+
+    def write(self, data):
+        data = np.ascontiguousarray(data)
+        _call(lib().galois_host_tensor_write(self.h, data.ctypes.data_as(C.c_void_p), data.nbytes))
+
+    def data_ptr(self):
+        return lib().galois_host_tensor_data(self.h)
+
     def to_cpu_tensor(self):
         """Host copy as a numpy array shaped [ne3..ne0] (row-major), uint8 block bytes for Q4_0."""
         nb = lib().galois_host_tensor_nbytes(self.h)
@@ -141,3 +172,94 @@ def galois_rope_custom(op, src0, src1, dst):
 
 def galois_soft_max(src, dst):
     _call(lib().galois_host_soft_max(src.h, dst.h))
+
+
+def galois_add(a, b, dst):
+    _call(lib().galois_host_add(a.h, b.h, dst.h))
+
+
+def galois_mul(a, b, dst):
+    _call(lib().galois_host_mul(a.h, b.h, dst.h))
+
+
+def galois_unary_silu(src, dst):
+    """``galois_unary(src, dst, UnaryOp::Silu)``."""
+    _call(lib().galois_host_unary_silu(src.h, dst.h))
+
+
+def galois_scale(src0, src1, dst):
+    _call(lib().galois_host_scale(src0.h, src1.h, dst.h))
+
+
+def galois_cpy(src, dst):
+    _call(lib().galois_host_cpy(src.h, dst.h))
+
+
+def galois_cont(src, dst):
+    _call(lib().galois_host_cont(src.h, dst.h))
+
+
+def galois_get_rows(src0, src1, dst):
+    _call(lib().galois_host_get_rows(src0.h, src1.h, dst.h))
+
+
+class LlamaDecoder:
+    """One-token decode step of a LLaMA-architecture model issued as galois ops (galois_amd/host/llama.hpp)."""
+
+    def __init__(self, device, n_vocab=32000, n_embd=4096, n_head=32, n_layer=32, n_ff=11008, n_ctx=2048,
+                 rms_eps=1e-6, freq_base=10000.0):
+        self.device = device
+        self.hp = dict(n_vocab=n_vocab, n_embd=n_embd, n_head=n_head, n_layer=n_layer, n_ff=n_ff, n_ctx=n_ctx,
+                       rms_eps=rms_eps, freq_base=freq_base)
+        self.h = lib().galois_host_llama_new(device.h, n_vocab, n_embd, n_head, n_layer, n_ff, n_ctx, rms_eps,
+                                             freq_base)
+        if not self.h:
+            _raise(3)
+
+    def close(self):
+        if self.h:
+            lib().galois_host_llama_free(self.h)
+            self.h = None
+
+    def tensor(self, name, layer=-1):
+        """Borrowed handle to a weight or cache tensor (owned by the decoder)."""
+        h = lib().galois_host_llama_tensor(self.h, name.encode(), layer)
+        if not h:
+            _raise(4)
+        hp = self.hp
+        e, f, v, c = hp["n_embd"], hp["n_ff"], hp["n_vocab"], hp["n_ctx"]
+        shapes = {"tok_embd": ((e, v), Q4_0), "output": ((e, v), Q4_0), "out_norm": ((e,), F32),
+                  "attn_norm": ((e,), F32), "ffn_norm": ((e,), F32), "wq": ((e, e), Q4_0), "wk": ((e, e), Q4_0),
+                  "wv": ((e, e), Q4_0), "wo": ((e, e), Q4_0), "w_gate": ((e, f), Q4_0), "w_up": ((e, f), Q4_0),
+                  "w_down": ((f, e), Q4_0), "k_cache": ((e, c), F32), "v_cache": ((e, c), F32)}
+        shape, dtype = shapes[name]
+        t = Tensor(h, shape, dtype)
+        t.borrowed = True
+        return t
+
+    def decode(self, token, n_past, fused=False):
+        _call(lib().galois_host_llama_decode(self.h, token, n_past, int(fused)))
+
+    def capture(self, token, n_past, fused=False):
+        _call(lib().galois_host_llama_capture(self.h, token, n_past, int(fused)))
+
+    def replay(self):
+        _call(lib().galois_host_llama_replay(self.h))
+
+    def logits(self):
+        t = Tensor(lib().galois_host_llama_logits(self.h), (self.hp["n_vocab"], 1), F32)
+        t.borrowed = True
+        return t.to_cpu_tensor().reshape(-1)
+
+    def ops_per_step(self):
+        return lib().galois_host_llama_ops_per_step(self.h)
+
+    def time_replays(self, n):
+        ms = C.c_float()
+        _call(lib().galois_host_llama_time_replays(self.h, self.device.h, n, C.byref(ms)))
+        return ms.value
+
+    def time_steps(self, token, n_past, fused, n):
+        ms = C.c_float()
+        _call(lib().galois_host_llama_time_steps(self.h, self.device.h, token, n_past, int(fused), n, C.byref(ms)))
+        return ms.value

@@ -45,6 +45,7 @@ extern "C" {
 
 typedef struct galois_hip_ctx galois_hip_ctx;
 typedef struct galois_hip_event galois_hip_event;
+typedef struct galois_hip_graph galois_hip_graph;
 
 /* ---- device / stream / buffer layer -------------------------------------- */
 
@@ -85,6 +86,16 @@ int32_t galois_hip_event_record(galois_hip_ctx *ctx, galois_hip_event *ev);
 int32_t galois_hip_event_elapsed_ms(galois_hip_ctx *ctx, galois_hip_event *start, galois_hip_event *stop,
                                     float *ms); /* synchronises on `stop` */
 int32_t galois_hip_event_destroy(galois_hip_ctx *ctx, galois_hip_event *ev);
+
+/* Stream capture (no counterpart in the reference, which launches every op of a decode step on its
+ * own: src/cuda.rs:476-565).  Ops issued on the context between begin and end are recorded instead of
+ * run; graph_launch replays them in order on the context's stream with the pointers and sizes they were
+ * recorded with.  While a capture is open, calls that allocate, free or block return
+ * GALOIS_HIP_E_UNSUPPORTED (a prefill matmul must have sized its workspace in an earlier eager call). */
+int32_t galois_hip_graph_begin_capture(galois_hip_ctx *ctx);
+int32_t galois_hip_graph_end_capture(galois_hip_ctx *ctx, galois_hip_graph **out);
+int32_t galois_hip_graph_launch(galois_hip_ctx *ctx, galois_hip_graph *graph);
+int32_t galois_hip_graph_destroy(galois_hip_ctx *ctx, galois_hip_graph *graph);
 
 /* ---- Q4_0 format ----------------------------------------------------------- */
 

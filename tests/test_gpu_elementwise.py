@@ -117,3 +117,44 @@ def test_elementwise_argument_errors(dev):
         with pytest.raises(GaloisHipError) as ei:
             call()
         assert ei.value.status == code
+
+
+@pytest.mark.parametrize("K,N,ne02,ne12,batch_fastest", [(128, 2048, 32, 32, True), (128, 37, 4, 4, True),
+                                                         (64, 50, 1, 3, False), (32, 7, 2, 2, False),
+                                                         (256, 19, 1, 1, False), (128, 21, 2, 6, True)])
+def test_decode_scores_kernel_shapes(dev, K, N, ne02, ne12, batch_fastest):
+    """M == 1 with rows contiguous along K: ragged row counts, both row orders, broadcast of a over the batch."""
+    rng = np.random.default_rng(K + N)
+    if batch_fastest:      # cache layout [N][ne02 * K]: batch stride K, row stride ne02 * K
+        store = rng.standard_normal((N, ne02 * K)).astype(np.float32)
+        a_view = np.lib.stride_tricks.as_strided(store, (ne02, N, K), (K * 4, ne02 * K * 4, 4))
+        s1, s2 = ne02 * K, K
+    else:
+        store = rng.standard_normal((ne02, N, K)).astype(np.float32)
+        a_view, s1, s2 = store, K, N * K
+    b = rng.standard_normal((ne12, 1, K)).astype(np.float32)
+    ab, bb, ob = dev.upload(store), dev.upload(b), _out(dev, ne12 * N)
+    dev.mul_mat_f32(ab, bb, ob, K, N, 1, ne02, ne12, 1, s1, s2)
+    emax, _ = npref.rel_err(dev.download(ob, np.float32, (ne12, 1, N)), oracle.mul_mat_f32(a_view, b))
+    assert emax < 1e-5
+
+
+@pytest.mark.parametrize("K,N,ne02,ne12", [(2048, 128, 32, 32), (1, 128, 2, 2), (15, 128, 2, 2), (17, 64, 1, 3),
+                                           (63, 100, 3, 3), (64, 100, 3, 3), (65, 100, 3, 3), (5000, 36, 2, 4),
+                                           (300, 4, 1, 1)])
+def test_decode_values_kernel_shapes(dev, K, N, ne02, ne12):
+    """M == 1 with a contiguous along N: one slab and many, ragged K, column tiles that end inside a wave,
+    broadcast of a over the batch; launched twice so the second run meets the tickets the first one left."""
+    rng = np.random.default_rng(K * 7 + N)
+    store = rng.standard_normal((K, ne02 * N)).astype(np.float32)           # cache layout [K][ne02 * N]
+    a_view = np.lib.stride_tricks.as_strided(store, (ne02, N, K), (N * 4, 4, ne02 * N * 4))
+    ab, ob = dev.upload(store), _out(dev, ne12 * N)
+    for rep in range(2):
+        b = rng.standard_normal((ne12, 1, K)).astype(np.float32)
+        bb = dev.upload(b)
+        dev.mul_mat_f32(ab, bb, ob, K, N, 1, ne02, ne12, ne02 * N, 1, N)
+        got = dev.download(ob, np.float32, (ne12, 1, N))
+        emax, _ = npref.rel_err(got, oracle.mul_mat_f32(a_view, b))
+        assert emax < 1e-5, rep
+        dev.mul_mat_f32(ab, bb, ob, K, N, 1, ne02, ne12, ne02 * N, 1, N)
+        assert np.array_equal(dev.download(ob, np.float32, (ne12, 1, N)), got)      # same bits every launch

@@ -1,0 +1,179 @@
+"""The LLaMA decode step issued as galois ops (galois_amd/host/llama.cpp) against the same sequence on the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle
+from galois_amd import host_api as g
+from tests import npref
+
+pytestmark = pytest.mark.gpu
+
+LAYER_Q = ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")
+
+
+def _make_weights(rng, hp):
+    e, f, v = hp["n_embd"], hp["n_ff"], hp["n_vocab"]
+    shapes = {"wq": (e, e), "wk": (e, e), "wv": (e, e), "wo": (e, e), "w_gate": (f, e), "w_up": (f, e), "w_down": (e, f)}
+
+    def q(rows, cols):
+        return oracle.quantize_q4_0((rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+
+    w = {"tok_embd": q(v, e), "output": q(v, e), "out_norm": (1 + 0.1 * rng.standard_normal(e)).astype(np.float32),
+         "layers": []}
+    for _ in range(hp["n_layer"]):
+        lw = {n: q(*shapes[n]) for n in LAYER_Q}
+        lw["attn_norm"] = (1 + 0.1 * rng.standard_normal(e)).astype(np.float32)
+        lw["ffn_norm"] = (1 + 0.1 * rng.standard_normal(e)).astype(np.float32)
+        w["layers"].append(lw)
+    return w
+
+
+def _load(dec, w, kc=None, vc=None):
+    for n in ("tok_embd", "output", "out_norm"):
+        dec.tensor(n).write(w[n])
+    for i, lw in enumerate(w["layers"]):
+        for n, a in lw.items():
+            dec.tensor(n, i).write(a)
+        if kc is not None:
+            dec.tensor("k_cache", i).write(kc[i])
+            dec.tensor("v_cache", i).write(vc[i])
+
+
+def _ref_step(w, hp, kc, vc, token, n_past):
+    """One token through the oracle's ops; kc / vc [n_layer][n_ctx][n_embd] are updated in place."""
+    e, h = hp["n_embd"], hp["n_head"]
+    d, L, eps = e // h, n_past + 1, hp["rms_eps"]
+    theta_scale = np.float32(hp["freq_base"]) ** np.float32(-2.0 / d)
+    pos = np.array([n_past], np.int32)
+    x = oracle.get_rows_q4_0(w["tok_embd"], np.array([token], np.int32))[0]
+    for i, lw in enumerate(w["layers"]):
+        a = oracle.mul(oracle.rms_norm(x, eps), lw["attn_norm"])
+        q, k, v = (oracle.mul_mat_q4_0_f32(lw[n], a) for n in ("wq", "wk", "wv"))
+        qr = oracle.rope(q.reshape(h, d), pos, 1.0, h, float(theta_scale))
+        kr = oracle.rope(k.reshape(h, d), pos, 1.0, h, float(theta_scale))
+        kc[i][n_past], vc[i][n_past] = kr.reshape(-1), v
+        kview = np.lib.stride_tricks.as_strided(kc[i], (h, L, d), (d * 4, e * 4, 4))
+        s = oracle.mul_mat_f32(kview, qr.reshape(h, 1, d))                       # [h, 1, L]
+        p = oracle.soft_max(oracle.scale(s, float(np.float32(1.0) / np.sqrt(np.float32(d)))).reshape(h, L))
+        vview = np.lib.stride_tricks.as_strided(vc[i], (h, d, L), (d * 4, 4, e * 4))
+        o = oracle.mul_mat_f32(vview, p.reshape(h, 1, L)).reshape(-1)            # [h, 1, d] -> [e]
+        x1 = oracle.add(oracle.mul_mat_q4_0_f32(lw["wo"], o), x)
+        f = oracle.mul(oracle.rms_norm(x1, eps), lw["ffn_norm"])
+        hh = oracle.mul(oracle.silu(oracle.mul_mat_q4_0_f32(lw["w_gate"], f)), oracle.mul_mat_q4_0_f32(lw["w_up"], f))
+        x = oracle.add(oracle.mul_mat_q4_0_f32(lw["w_down"], hh), x1)
+    return oracle.mul_mat_q4_0_f32(w["output"], oracle.mul(oracle.rms_norm(x, eps), w["out_norm"]))
+
+
+SMALL = dict(n_vocab=512, n_embd=256, n_head=2, n_layer=2, n_ff=512, n_ctx=64, rms_eps=1e-6, freq_base=10000.0)
+
+
+@pytest.fixture(scope="module")
+def gdev():
+    return g.Device.gpu(0)
+
+
+def _check(got, ref, tol):
+    emax, el2 = npref.rel_err(got, ref)
+    assert emax < tol and el2 < tol, (emax, el2)
+
+
+def test_decode_step_matches_oracle_with_a_filled_cache(gdev):
+    rng = np.random.default_rng(50)
+    hp = SMALL
+    w = _make_weights(rng, hp)
+    n_past = 37
+    kc = rng.standard_normal((hp["n_layer"], hp["n_ctx"], hp["n_embd"])).astype(np.float32)
+    vc = rng.standard_normal((hp["n_layer"], hp["n_ctx"], hp["n_embd"])).astype(np.float32)
+    dec = g.LlamaDecoder(gdev, **hp)
+    _load(dec, w, kc, vc)
+    ref = _ref_step(w, hp, kc.copy(), vc.copy(), 123, n_past)
+    for fused in (False, True):
+        _load(dec, w, kc, vc)
+        dec.decode(123, n_past, fused)
+        _check(dec.logits(), ref, 1e-4)
+    assert dec.ops_per_step() == 1 + hp["n_layer"] * 20 + 2      # fused: 20 launches per layer
+    # the step wrote row n_past of both caches and nothing else
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    _ref_step(w, hp, kc_ref, vc_ref, 123, n_past)
+    for i in range(hp["n_layer"]):
+        kg = dec.tensor("k_cache", i).to_cpu_tensor()
+        vg = dec.tensor("v_cache", i).to_cpu_tensor()
+        rows = np.arange(hp["n_ctx"]) != n_past
+        assert np.array_equal(kg[rows], kc[i][rows]) and np.array_equal(vg[rows], vc[i][rows])
+        _check(kg[n_past], kc_ref[i][n_past], 1e-4)
+        _check(vg[n_past], vc_ref[i][n_past], 1e-4)
+    dec.close()
+
+
+def test_decode_from_an_empty_cache_over_several_tokens(gdev):
+    rng = np.random.default_rng(51)
+    hp = SMALL
+    w = _make_weights(rng, hp)
+    dec = g.LlamaDecoder(gdev, **hp)
+    _load(dec, w)
+    kc = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float32)
+    vc = np.zeros_like(kc)
+    for n_past, tok in enumerate([1, 400, 17, 17, 511]):
+        ref = _ref_step(w, hp, kc, vc, tok, n_past)
+        dec.decode(tok, n_past, False)
+        _check(dec.logits(), ref, 1e-4)
+    dec.close()
+
+
+def test_graph_replays_equal_the_eager_step(gdev):
+    rng = np.random.default_rng(52)
+    hp = SMALL
+    w = _make_weights(rng, hp)
+    kc = rng.standard_normal((hp["n_layer"], hp["n_ctx"], hp["n_embd"])).astype(np.float32)
+    dec = g.LlamaDecoder(gdev, **hp)
+    _load(dec, w, kc, kc[::-1].copy())
+    dec.decode(9, 20, True)
+    eager = dec.logits()
+    dec.capture(9, 20, True)
+    for i in range(4):
+        dec.replay()
+        assert np.array_equal(dec.logits(), eager), i
+        # eager work and synchronisation between the replays
+        dec.decode(9 + i, 30 + i, False)        # appends rows the recorded step (21 keys) never reads
+        assert not np.array_equal(dec.logits(), eager)
+        dec.decode(9, 20, True)                 # puts token 9 / position 20 back into the device-side inputs
+    dec.close()
+
+
+def test_capture_refuses_calls_that_allocate_or_block(dev):
+    from galois_amd import GaloisHipError
+    x = dev.upload(np.arange(8, dtype=np.float32))
+    y = dev.alloc(32)
+    dev.graph_begin_capture()
+    try:
+        for call in (lambda: dev.alloc(64), dev.synchronize, lambda: dev.download(x, np.float32, 8),
+                     dev.graph_begin_capture):
+            with pytest.raises(GaloisHipError) as ei:
+                call()
+            assert ei.value.status == -5
+        dev.scale_f32(x, y, 2.0, 8)
+    finally:
+        graph = dev.graph_end_capture()
+    assert np.array_equal(dev.download(y, np.float32, 8), np.zeros(8, np.float32))      # recorded, not run
+    dev.graph_launch(graph)
+    assert np.array_equal(dev.download(y, np.float32, 8), 2 * np.arange(8, dtype=np.float32))
+    dev.graph_destroy(graph)
+
+
+def test_full_width_layer_at_kv_length_2048(gdev):
+    """One layer at LLaMA-7B width (4096 / 32 heads / 11008 / vocab 32000) attending over 2048 cached positions."""
+    rng = np.random.default_rng(53)
+    hp = dict(n_vocab=32000, n_embd=4096, n_head=32, n_layer=1, n_ff=11008, n_ctx=2048, rms_eps=1e-6,
+              freq_base=10000.0)
+    w = _make_weights(rng, hp)
+    kc = rng.standard_normal((1, 2048, 4096)).astype(np.float32)
+    vc = rng.standard_normal((1, 2048, 4096)).astype(np.float32)
+    dec = g.LlamaDecoder(gdev, **hp)
+    _load(dec, w, kc, vc)
+    ref = _ref_step(w, hp, kc, vc, 31999, 2047)
+    dec.decode(31999, 2047, False)
+    _check(dec.logits(), ref, 1e-4)
+    dec.capture(31999, 2047, True)
+    dec.replay()
+    _check(dec.logits(), ref, 1e-4)
+    dec.close()
