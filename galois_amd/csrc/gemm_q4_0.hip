@@ -124,35 +124,54 @@ __global__ __launch_bounds__(256) void gemm_q4_0_mfma_v1(const uint8_t *__restri
 // ---------------------------------------------------------------------------------------
 // Main kernel: K % 256 == 0, W and X 16-byte aligned.
 //
-//   - X is rounded to fp16 once by f32_to_f16_rows into a context-owned workspace, so a
-//     tile row of 64 k-values is one 128-byte line and the 4 MB panel stays L2-resident.
-//   - Workgroup tile 128 (M) x 176 (N), k-step 64 (two Q4_0 blocks = one 36-byte slot per
-//     weight row, fetched with dwordx4 + dwordx4 + dword).  11008 = 62.5 x 176, so the
-//     512 x 11008 prefill is 4 x 63 = 252 workgroups: one round on 256 CUs.
-//   - 8 waves: 4 consumers as 2 (M) x 2 (N), wave tile 64 x 96 or 64 x 80 -> 4 x 6 (or 5)
-//     tiles of v_mfma_f32_16x16x32_f16 with f32 accumulators in registers, and 4 producers
-//     that load, dequantise and store; each SIMD hosts one wave of each kind.
-//   - LDS double-buffered: while MFMA consumes stage s the producers fill the other buffer
-//     with stage s+1 and have stages s+2, s+3 in flight from memory; one barrier per stage.
+//   - X is rounded to fp16 once by f32_to_f16_tiles into a context-owned workspace, stored in the
+//     order the A operand of v_mfma_f32_16x16x32_f16 is held (per lane 8 consecutive k of one row),
+//     so a fragment is one contiguous KB: the consumer waves fetch their A fragments straight from
+//     global memory (the 4 MB panel stays in L2) one stage ahead, and X never touches LDS.
+//   - Workgroup tile 128 (M) x 176 (N), k-stage 64 (two Q4_0 blocks = one 36-byte slot per weight
+//     row).  11008 = 62.5 x 176, so the 512 x 11008 prefill is 4 x 63 = 252 workgroups: one round
+//     on 256 CUs.
+//   - 8 waves: 4 consumers as 2 (M) x 2 (N), wave tile 64 x 96 or 64 x 80 -> 4 x 6 (or 5) MFMA
+//     tiles with f32 accumulators in registers, and 4 producers that fetch the weights as whole
+//     144-byte row pieces (4 stages at a time), park them raw in LDS, and each stage dequantise
+//     one slot per row into an fp16 B tile.  Each SIMD hosts one wave of each kind.
+//   - The fp16 B tile is triple-buffered, one barrier per stage: while the consumers multiply the
+//     second k-half of stage s they already hold the first half of stage s+1, and the producers
+//     write stage s+2.  LDS carries only B: 22 KB of fragment reads and 11 KB of writes per 32 k
+//     against 384 MFMA cycles per SIMD.
 //   - blockIdx is mapped so that an XCD (blockIdx % 8) owns one 128-row panel of X and a
 //     contiguous range of weight tiles: X stays in that XCD's L2, W streams once per panel.
 constexpr int GM = 128, GN = 176, GK = 64;
-constexpr int GSTRIDE = 72;                 // halfs per LDS row: 144-byte rows -> conflict-free 16-byte reads
-constexpr int GA_HALFS = GM * GSTRIDE;      // 9216 halfs  (18,432 B)
-constexpr int GB_HALFS = GN * GSTRIDE;      // 12672 halfs (25,344 B)
+constexpr int GBSTRIDE = 80;                  // halfs per B row in LDS: 160-byte rows
+constexpr int GB_HALFS = GN * GBSTRIDE;       // 14,080 halfs (28,160 B) per stage buffer
+constexpr int GNBUF = 3;
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void f32_to_f16_rows(const float *__restrict__ x, _Float16 *__restrict__ y,
-                                                       int64_t n8) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n8) return;
-    const float4 a = reinterpret_cast<const float4 *>(x)[2 * i], b = reinterpret_cast<const float4 *>(x)[2 * i + 1];
-    uint4 o;
-    o.x = pack_h2(a.x, a.y), o.y = pack_h2(a.z, a.w), o.z = pack_h2(b.x, b.y), o.w = pack_h2(b.z, b.w);
-    reinterpret_cast<uint4 *>(y)[i] = o;
+// X -> fp16 in the order the MFMA A operand is fetched: tiles of 16 rows x 32 k (1 KB), tile (m16, kb)
+// at ((m16 * K/32) + kb) * 1 KB, and inside a tile the 16-byte run k = kb*32 + kg*8 .. +7 of row
+// m16*16 + r at (kg * 16 + r) * 16 bytes.  Lane l = kg * 16 + r of a wave owns exactly that run in
+// v_mfma_f32_16x16x32_f16, so a fragment load is 64 consecutive 16-byte pieces: one contiguous KB.
+// Rows past M (the last tile of a ragged M) are written as zeros.
+__global__ __launch_bounds__(256) void f32_to_f16_tiles(const float *__restrict__ x, _Float16 *__restrict__ y, int M,
+                                                        int K, int64_t nchunks) {
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte output chunk
+    if (o >= nchunks) return;
+    const int64_t tile = o >> 6;
+    const int c = (int)(o & 63), kg = c >> 4, r = c & 15;
+    const int kblocks = K / 32;
+    const int64_t m16 = tile / kblocks;
+    const int kb = (int)(tile - m16 * kblocks);
+    const int64_t m = m16 * 16 + r;
+    uint4 out = make_uint4(0, 0, 0, 0);
+    if (m < M) {
+        const float4 *src = reinterpret_cast<const float4 *>(x + m * K + kb * 32 + kg * 8);
+        const float4 a = src[0], b = src[1];
+        out.x = pack_h2(a.x, a.y), out.y = pack_h2(a.z, a.w), out.z = pack_h2(b.x, b.y), out.w = pack_h2(b.z, b.w);
+    }
+    reinterpret_cast<uint4 *>(y)[o] = out;
 }
 
-// Four nibble bytes (one dword of qs, already aligned) -> 4 + 4 fp16 weights:
+// Four nibble bytes (one dword of qs) -> 4 + 4 fp16 weights:
 // lo[0..1] = bytes 0..3 low nibbles (k = 4j .. 4j+3), hi[0..1] = high nibbles (k = 16+4j ..).
 // (1024 + n) - 1032 is the exact integer n - 8; the product with d is rounded once.
 __device__ __forceinline__ void deq_dword(uint32_t v, half2_t d2, uint32_t lo[2], uint32_t hi[2]) {
@@ -170,66 +189,25 @@ __device__ __forceinline__ void deq_dword(uint32_t v, half2_t d2, uint32_t lo[2]
     hi[1] = __builtin_bit_cast(uint32_t, (h23 - off) * d2);
 }
 
-// One Q4_0 block (d bits + 4 aligned qs dwords) -> 32 fp16 values written to an LDS row.
-__device__ __forceinline__ void deq_block_to_lds(uint32_t dbits, const uint32_t q[4], _Float16 *dst) {
-    const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t)dbits);
-    const half2_t d2 = {d, d};
-    uint32_t lo[8], hi[8];
-#pragma unroll
-    for (int j = 0; j < 4; j++) deq_dword(q[j], d2, lo + 2 * j, hi + 2 * j);
-    uint4 *p = reinterpret_cast<uint4 *>(dst);
-    p[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-    p[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-    p[2] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-    p[3] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-}
-
-// Producer side.  The upper 4 waves of the workgroup fetch and convert; the lower 4 waves only
-// read fragments and issue MFMA.  Every SIMD therefore hosts one wave of each kind and the
-// hardware overlaps the dequantisation arithmetic of one with the matrix instructions of the
-// other without any hand scheduling.
-//
-// All global loads are whole-line: eight consecutive lanes fetch the eight 16-byte chunks of one
-// 128-byte line of X; the weights are fetched four stages at a time as the 144 contiguous bytes
-// (8 blocks) each tile row contributes, parked as raw bytes in LDS, and every stage a thread
-// lifts its row's 36-byte slot back out, dequantises it and stores fp16.
+// ---- producer side ---------------------------------------------------------------------
+// The weights are fetched four stages at a time as the 144 contiguous bytes (8 blocks) each
+// tile row contributes: nine consecutive lanes read one row piece with 16-byte loads, so every
+// request is made of whole lines.  The pieces are parked as raw bytes in LDS.
 constexpr int GRAW_STRIDE = 144;                 // raw bytes per tile row per super-stage (4 slots)
 constexpr int GRAW_BYTES = GN * GRAW_STRIDE;     // 25,344 B per raw buffer
 constexpr int GRAW_CHUNKS = GN * 9;              // 16-byte chunks per raw buffer
 constexpr int GRAW_PER_THREAD = (GRAW_CHUNKS + 255) / 256;
+constexpr size_t GEMM_LDS_BYTES = (size_t)GNBUF * GB_HALFS * sizeof(_Float16) + 2 * (size_t)GRAW_BYTES + 16;
 
-// The producers' global loads are issued through inline assembly and waited for by hand.
-// Loads retire in order, so "at most n younger loads outstanding" is the exact condition for an
-// older load to have landed.  Left to the compiler, loads whose use is one or more loop
-// iterations away are waited for with vmcnt(0), which also drains every prefetch issued since.
+// Global loads whose use is a loop iteration (or four) away are issued through inline assembly and
+// waited for by hand: loads retire in order, so "at most n younger loads outstanding" is the exact
+// condition for an older one to have landed, whereas the compiler waits for such loads with vmcnt(0)
+// right where they are issued (or parks them in scratch memory).
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void gload16(u32x4_t &dst, const void *ptr) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
 }
 #define GEMM_VMWAIT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
-
-struct gemm_x_regs {
-    u32x4_t c[4];  // chunk j: row 32*j + p/8, 16-byte chunk p%8 of that row's 128-byte line
-};
-
-__device__ __forceinline__ void gemm_load_x(const _Float16 *xbase, int K, int M, int m0, int p, int s, gemm_x_regs &r) {
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int row = min(m0 + 32 * j + (p >> 3), M - 1);
-        gload16(r.c[j], xbase + (size_t)row * K + (size_t)s * GK + (p & 7) * 8);
-    }
-}
-
-__device__ __forceinline__ void gemm_store_x(_Float16 *As, int p, const gemm_x_regs &r) {
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-        *reinterpret_cast<u32x4_t *>(As + (32 * j + (p >> 3)) * GSTRIDE + (p & 7) * 8) = r.c[j];
-}
-
-__device__ __forceinline__ void gemm_keep_alive(const gemm_x_regs &r) {
-#pragma unroll
-    for (int j = 0; j < 4; j++) asm volatile("" ::"v"(r.c[j]));
-}
 
 struct gemm_raw_regs {
     u32x4_t c[GRAW_PER_THREAD];
@@ -239,8 +217,6 @@ __device__ __forceinline__ void gemm_load_raw(const uint8_t *W, size_t wrow_byte
                                               gemm_raw_regs &r) {
 #pragma unroll
     for (int i = 0; i < GRAW_PER_THREAD; i++) {
-        // unconditional (clamped) so that the number of loads in flight is the same on every path:
-        // the compiler can then wait for exactly the loads it needs instead of draining them all
         const int q = min(p + 256 * i, GRAW_CHUNKS - 1);
         const int row = q / 9, c = q - row * 9;
         gload16(r.c[i], W + (size_t)min(n0 + row, N - 1) * wrow_bytes + (size_t)super * GRAW_STRIDE + c * 16);
@@ -255,147 +231,205 @@ __device__ __forceinline__ void gemm_store_raw(uint8_t *raw, int p, const gemm_r
     }
 }
 
-// Slot J (0..3) of tile row `prow` out of a raw buffer: three aligned 16-byte reads cover the
-// 36 bytes at offset 36*J; dequantise both blocks into the fp16 B tile.
+// One stage of B: slot J (36 bytes) of every tile row out of a raw buffer, as 4 tasks per row:
+// task (b, jp) = eight nibble bytes qs[8*jp .. 8*jp+7] of block b -> the 16-byte run k = 32b + 8jp ..
+// (low nibbles) and the run k = 32b + 16 + 8jp .. (high nibbles).  The four lanes of a row write
+// 64 distinct bytes per store and neighbouring rows are 160 bytes apart, so the 16-byte stores of
+// eight consecutive lanes fall into 32 different banks.
 template <int J>
-__device__ __forceinline__ void gemm_dequant_slot(const uint8_t *raw, _Float16 *Bs, int prow) {
-    constexpr int first = (36 * J) / 16;        // first 16-byte piece
-    constexpr int skip = (36 * J) / 4 - 4 * first;  // dwords to skip inside it
-    const uint4 *src = reinterpret_cast<const uint4 *>(raw + prow * GRAW_STRIDE) + first;
-    const uint4 a = src[0], b = src[1], c = src[2];
-    const uint32_t d[12] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w, c.x, c.y, c.z, c.w};
-    uint32_t w[9];
+__device__ __forceinline__ void gemm_dequant_stage(const uint8_t *raw, _Float16 *Bs, int p) {
+#ifdef GEMM_X_NO_DEQ
+    return;
+#endif
+    // all LDS reads of the thread's (up to) three tasks first, so that their latencies overlap
+    uint32_t dbits[3], w0[3], w1[3], w2[3];
 #pragma unroll
-    for (int i = 0; i < 9; i++) w[i] = d[skip + i];
-    // block A: qs bytes straddle the slot's dwords by two bytes; block B is aligned
-    const uint32_t qa[4] = {__builtin_amdgcn_alignbit(w[1], w[0], 16), __builtin_amdgcn_alignbit(w[2], w[1], 16),
-                            __builtin_amdgcn_alignbit(w[3], w[2], 16), __builtin_amdgcn_alignbit(w[4], w[3], 16)};
-    deq_block_to_lds(w[0] & 0xFFFFu, qa, Bs + prow * GSTRIDE);
-    const uint32_t qb[4] = {w[5], w[6], w[7], w[8]};
-    deq_block_to_lds(w[4] >> 16, qb, Bs + prow * GSTRIDE + 32);
+    for (int it = 0; it < 3; it++) {
+        const int q = p + 256 * it;
+        if (it < 2 || q < GN * 4) {
+            const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
+            const int o = row * GRAW_STRIDE + 36 * J + 18 * b;  // the block: d at o, qs at o + 2
+            dbits[it] = *reinterpret_cast<const uint16_t *>(raw + o);
+            const int qo = o + 2 + 8 * jp;                       // 4-byte aligned for b = 1, 2 mod 4 for b = 0
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(raw + (qo & ~3));
+            w0[it] = w[0], w1[it] = w[1], w2[it] = w[2];         // w2 of the very last task lies in the 16-byte pad
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int it = 0; it < 3; it++) {
+        const int q = p + 256 * it;
+        if (it < 2 || q < GN * 4) {
+            const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
+            const uint32_t sh = b ? 0u : 16u;
+            const uint32_t q0 = __builtin_amdgcn_alignbit(w1[it], w0[it], sh);
+            const uint32_t q1 = __builtin_amdgcn_alignbit(w2[it], w1[it], sh);
+            const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t)dbits[it]);
+            const half2_t d2 = {d, d};
+            uint32_t lo[4], hi[4];
+            deq_dword(q0, d2, lo, hi);
+            deq_dword(q1, d2, lo + 2, hi + 2);
+            _Float16 *dst = Bs + row * GBSTRIDE + 32 * b + 8 * jp;
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            *reinterpret_cast<uint4 *>(dst + 16) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        }
+    }
 }
 
-// LDS map: [2] fp16 stage buffers (A | B), then [2] raw weight buffers.
-constexpr int GBUF_HALFS = GA_HALFS + GB_HALFS;
-constexpr size_t GEMM_LDS_BYTES = 2 * (size_t)GBUF_HALFS * sizeof(_Float16) + 2 * (size_t)GRAW_BYTES;
-
-__device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__restrict__ W,
-                                              const _Float16 *__restrict__ Xh, int K, int N, int M, int m0, int n0) {
+// Barrier protocol (both kinds of wave meet every one): R after the first raw piece is parked,
+// then barrier t after stage t is written, for t = 0 .. nslots-1.  Stage t goes to buffer t % 3.
+__device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__restrict__ W, int K, int N, int n0) {
     const int p = threadIdx.x - 256;
     const int nslots = K / 64;            // stages; a multiple of 4 (K % 256 == 0)
     const int nsuper = nslots / 4;
     const size_t wrow_bytes = (size_t)nslots * 36;
-    uint8_t *raw0 = reinterpret_cast<uint8_t *>(smem + 2 * GBUF_HALFS);
+    uint8_t *raw0 = reinterpret_cast<uint8_t *>(smem + GNBUF * GB_HALFS);
     uint8_t *raw1 = raw0 + GRAW_BYTES;
-    const bool has_w = p < GN;
 
-    // prologue: raw super-stage 0 parked, super-stage 1 requested; X stages 0..3 requested
     gemm_raw_regs rr;
-    gemm_x_regs x0, x1, x2, x3;  // X ring: stage t lives in x[t % 4]
     gemm_load_raw(W, wrow_bytes, N, n0, p, 0, rr);
-    gemm_load_x(Xh, K, M, m0, p, 0, x0);
-    gemm_load_x(Xh, K, M, m0, p, 1, x1);
-    gemm_load_x(Xh, K, M, m0, p, 2, x2);
-    gemm_load_x(Xh, K, M, m0, p, 3, x3);
-    static_assert(GRAW_PER_THREAD == 7, "the hand-written vmcnt values below count 7 raw + 4 X loads per batch");
-    GEMM_VMWAIT(16);  // raw super-stage 0 landed (16 younger X loads may still fly)
+    GEMM_VMWAIT(0);
     gemm_store_raw(raw0, p, rr);
     gemm_load_raw(W, wrow_bytes, N, n0, p, min(1, nsuper - 1), rr);
-    __syncthreads();  // raw0 visible to every producer
-    GEMM_VMWAIT(19);  // x0 landed (younger: x1..x3 and one raw batch)
-    gemm_store_x(smem, p, x0);
-    if (has_w) gemm_dequant_slot<0>(raw0, smem + GA_HALFS, p);
-    gemm_load_x(Xh, K, M, m0, p, min(4, nslots - 1), x0);
-    __syncthreads();  // stage 0 visible to the consumers
-
-    // Step run while the consumers compute stage S: produce stage t = S+1 (slot J = t % 4 of its
-    // super-stage) into buffer t&1 from X ring register XR, then request X stage t+4 into XR.
-    // On the last slot of a super-stage the raw bytes of the next one (requested four stages
-    // ago) are parked in the other raw buffer, whose previous content was last read long before,
-    // and the one after that is requested.
-#define GEMM_PRODUCE(S, J, XR)                                                                   \
-    {                                                                                            \
-        const int t = (S) + 1;                                                                   \
-        const int sup = t >> 2;                                                                  \
-        _Float16 *buf = smem + (t & 1) * GBUF_HALFS;                                             \
-        GEMM_VMWAIT(19); /* XR was requested four steps ago: 3 x 4 X loads + 7 raw loads younger */ \
-        gemm_store_x(buf, p, XR);                                                                \
-        if (has_w) gemm_dequant_slot<J>((sup & 1) ? raw1 : raw0, buf + GA_HALFS, p);             \
-        gemm_load_x(Xh, K, M, m0, p, min(t + 4, nslots - 1), XR);                                \
-        if ((J) == 3) {                                                                          \
-            GEMM_VMWAIT(16); /* rr was requested four steps ago: 4 x 4 X loads younger */        \
-            gemm_store_raw(((sup + 1) & 1) ? raw1 : raw0, p, rr);                                \
-            gemm_load_raw(W, wrow_bytes, N, n0, p, min(sup + 2, nsuper - 1), rr);                \
-        }                                                                                        \
-        __syncthreads();                                                                         \
+    __syncthreads();  // R
+    for (int sup = 0; sup < nsuper; sup++) {
+        const uint8_t *raw = (sup & 1) ? raw1 : raw0;
+        const int t = 4 * sup;
+        gemm_dequant_stage<0>(raw, smem + (t % GNBUF) * GB_HALFS, p);
+        __syncthreads();
+        gemm_dequant_stage<1>(raw, smem + ((t + 1) % GNBUF) * GB_HALFS, p);
+        __syncthreads();
+        gemm_dequant_stage<2>(raw, smem + ((t + 2) % GNBUF) * GB_HALFS, p);
+        __syncthreads();
+        gemm_dequant_stage<3>(raw, smem + ((t + 3) % GNBUF) * GB_HALFS, p);
+        // park the next piece (requested four stages ago) in the other raw buffer, whose last readers
+        // passed a barrier three stages ago, and request the one after it
+        GEMM_VMWAIT(0);
+        gemm_store_raw((sup & 1) ? raw0 : raw1, p, rr);
+        gemm_load_raw(W, wrow_bytes, N, n0, p, min(sup + 2, nsuper - 1), rr);
+        __syncthreads();
     }
-    // full groups of four steps: no conditionals, so every load has a fixed distance to its use
-    int s = 0;
-    for (; s + 4 < nslots; s += 4) {
-        GEMM_PRODUCE(s, 1, x1)
-        GEMM_PRODUCE(s + 1, 2, x2)
-        GEMM_PRODUCE(s + 2, 3, x3)
-        GEMM_PRODUCE(s + 3, 0, x0)
-    }
-    // last group: stages nslots-3 .. nslots-1 are produced, the final step only meets the barrier
-    // (the J == 3 step parks a clamped, unused copy of the last super-stage: harmless)
-    GEMM_PRODUCE(s, 1, x1)
-    GEMM_PRODUCE(s + 1, 2, x2)
-    GEMM_PRODUCE(s + 2, 3, x3)
-    __syncthreads();
-    // The last requests of every ring register are never consumed.  To the compiler an inline-asm
-    // load defines its destination at once, so a dead destination could be handed to some other
-    // value while the load is still in flight and be overwritten when it lands.  Drain the loads,
-    // then name every ring register once more so that all of them stay allocated until here.
+    // The last request is never consumed.  To the compiler an inline-asm load defines its destination at
+    // once, so a dead destination could be handed to another value while the load is still in flight and
+    // be overwritten when it lands.  Drain, then name every register so all stay allocated until here.
     GEMM_VMWAIT(0);
-    gemm_keep_alive(x0);
-    gemm_keep_alive(x1);
-    gemm_keep_alive(x2);
-    gemm_keep_alive(x3);
 #pragma unroll
     for (int i = 0; i < GRAW_PER_THREAD; i++) asm volatile("" ::"v"(rr.c[i]));
-#undef GEMM_PRODUCE
 }
 
-// Consumer side: a wave that owns NF 16-wide column tiles starting at ncol0 and rows wm*64..+63.
+// ---- consumer side -----------------------------------------------------------------------
+// The A fragments are requested through inline assembly and waited for by hand.  Loads retire in
+// order, so "at most 8 younger loads outstanding" is the exact condition for the previous stage's
+// eight to have landed; left to the compiler, a load whose use is a loop iteration away is waited
+// for with vmcnt(0), which would also drain the prefetch just issued.
+struct gemm_a_regs {
+    u32x4_t c[8];  // [ks * 4 + i]: rows i*16 + lane%16 of the wave's 64, k = ks*32 + (lane/16)*8 ..
+};
+
+// Address = scalar base (the panel advanced to the stage: 2 KB per stage) + per-lane 32-bit offset
+// of the lane's piece in the first k-block of its 16-row group + immediate (second k-block: + 1 KB).
+__device__ __forceinline__ void gemm_load_a(gemm_a_regs &r, const _Float16 *xs, const uint32_t (&ro)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r.c[i]) : "v"(ro[i]), "s"(xs) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(r.c[4 + i]) : "v"(ro[i]), "s"(xs) : "memory");
+    }
+}
+
+// Waits until at most N loads are outstanding; naming the registers makes every later use of
+// them depend on the wait.
+#ifdef GEMM_X_HALF_A
+#define GEMM_WAIT_A(N, r) GEMM_WAIT_A_(4, r)
+#else
+#define GEMM_WAIT_A(N, r) GEMM_WAIT_A_(N, r)
+#endif
+#define GEMM_WAIT_A_(N, r)                                                                                   \
+    asm volatile("s_waitcnt vmcnt(" #N ")"                                                                   \
+                 : "+v"((r).c[0]), "+v"((r).c[1]), "+v"((r).c[2]), "+v"((r).c[3]), "+v"((r).c[4]), "+v"((r).c[5]), \
+                   "+v"((r).c[6]), "+v"((r).c[7])::"memory")
+
+#ifdef GEMM_X_NO_A
+#define GEMM_XA(...)
+#else
+#define GEMM_XA(...) __VA_ARGS__
+#endif
+#ifdef GEMM_X_NO_MFMA
+#define GEMM_MFMA(a, b, c) (c)
+#else
+#define GEMM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
+#endif
+#ifdef GEMM_X_NO_MFMA
+#define GEMM_XKEEP _Pragma("unroll") for (int j = 0; j < NF; j++) { asm volatile("" ::"v"(b0[j]), "v"(b1[j])); }
+#else
+#define GEMM_XKEEP
+#endif
 template <int NF>
-__device__ __forceinline__ void gemm_consumer(const _Float16 *smem, float *__restrict__ Y, int K, int N, int M, int m0,
-                                              int n0, int wm, int ncol0) {
+__device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float16 *__restrict__ Xh,
+                                              float *__restrict__ Y, int K, int N, int M, int m0, int n0, int wm,
+                                              int ncol0) {
     const int lane = threadIdx.x & 63;
     const int nslots = K / 64;
-    constexpr int BUF = GBUF_HALFS;
     float4_t acc[4][NF];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < NF; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
-    const int a_off = (wm * 64 + (lane & 15)) * GSTRIDE + (lane >> 4) * 8;
-    const int b_off = GA_HALFS + (ncol0 + (lane & 15)) * GSTRIDE + (lane >> 4) * 8;
-    __syncthreads();  // producers: raw weights parked
-    __syncthreads();  // producers: stage 0 ready
-    for (int s = 0; s < nslots; s++) {
-        const _Float16 *buf = smem + (s & 1) * BUF;
-        // both k-halves of the stage are requested up front so the second half's LDS latency
-        // hides behind the first half's matrix instructions
-        half8_t a[2][4], b[2][NF];
+    uint32_t ro[4];  // byte offsets in the tiled panel (the host checks that the panel is below 4 GB)
+    const int m16_last = (M + 15) / 16 - 1;
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+    for (int i = 0; i < 4; i++)
+        ro[i] = (uint32_t)min(m0 / 16 + wm * 4 + i, m16_last) * (uint32_t)(K / 32) * 1024u + lane * 16u;
+    const int b_off = (ncol0 + (lane & 15)) * GBSTRIDE + (lane >> 4) * 8;
+
+    gemm_a_regs a0, a1;
+    GEMM_XA(gemm_load_a(a0, Xh, ro);)
+    half8_t b0[NF], b1[NF];
+    __syncthreads();  // R
+    __syncthreads();  // stage 0 written
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                a[ks][i] = *reinterpret_cast<const half8_t *>(buf + a_off + i * 16 * GSTRIDE + ks * 32);
-#pragma unroll
-            for (int j = 0; j < NF; j++)
-                b[ks][j] = *reinterpret_cast<const half8_t *>(buf + b_off + j * 16 * GSTRIDE + ks * 32);
-        }
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < NF; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[ks][i], b[ks][j], acc[i][j], 0, 0, 0);
-        __syncthreads();
+    for (int j = 0; j < NF; j++) b0[j] = *reinterpret_cast<const half8_t *>(smem + b_off + j * 16 * GBSTRIDE);
+
+    // One stage: AC holds this stage's A fragments (requested a stage ago), AN receives the next.
+    // LAST drops what prepares a following stage.  cur / nxt are the LDS offsets of this stage's and
+    // the next stage's B buffers.
+    int cur = b_off, nxt = b_off + GB_HALFS;
+#define GEMM_STAGE(S, AC, AN, LAST)                                                                        \
+    {                                                                                                      \
+        GEMM_XA(if (!(LAST)) gemm_load_a(AN, Xh + ((S) + 1) * 1024, ro);)                                    \
+        if (LAST)                                                                                          \
+            GEMM_WAIT_A(0, AC);                                                                            \
+        else                                                                                               \
+            GEMM_WAIT_A(8, AC);                                                                            \
+        _Pragma("unroll") for (int j = 0; j < NF; j++)                                                     \
+            b1[j] = *reinterpret_cast<const half8_t *>(smem + cur + j * 16 * GBSTRIDE + 32);               \
+        __builtin_amdgcn_sched_barrier(0); /* keep the fragment reads ahead of the matrix instructions */  \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) _Pragma("unroll") for (int j = 0; j < NF; j++)       \
+            acc[i][j] = GEMM_MFMA(__builtin_bit_cast(half8_t, (AC).c[i]), b0[j], acc[i][j]);               \
+        __builtin_amdgcn_sched_barrier(0);                                                                 \
+        if (!(LAST)) {                                                                                     \
+            __syncthreads(); /* stage S+1 written */                                                       \
+            _Pragma("unroll") for (int j = 0; j < NF; j++)                                                 \
+                b0[j] = *reinterpret_cast<const half8_t *>(smem + nxt + j * 16 * GBSTRIDE);                \
+        }                                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                 \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) _Pragma("unroll") for (int j = 0; j < NF; j++)       \
+            acc[i][j] = GEMM_MFMA(__builtin_bit_cast(half8_t, (AC).c[4 + i]), b1[j], acc[i][j]);           \
+        GEMM_XKEEP                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                                 \
+        cur = nxt;                                                                                         \
+        nxt = (nxt == b_off + (GNBUF - 1) * GB_HALFS) ? b_off : nxt + GB_HALFS;                            \
     }
+    int s = 0;
+    for (; s < nslots - 2; s += 2) {
+        GEMM_STAGE(s, a0, a1, false)
+        GEMM_STAGE(s + 1, a1, a0, false)
+    }
+    GEMM_STAGE(s, a0, a1, false)
+    GEMM_STAGE(s + 1, a1, a0, true)
+#undef GEMM_STAGE
+
+    // every A request has been waited for: the last stage drained the counter
+
     // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -413,7 +447,7 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, float *__res
 __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict__ W, const _Float16 *__restrict__ Xh,
                                                       float *__restrict__ Y, int K, int N, int M, int n_tiles,
                                                       int m_tiles) {
-    extern __shared__ __attribute__((aligned(16))) _Float16 smem[];  // [2][A | B]
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[];  // [3] B stage | [2] raw | pad
     // XCD-aware tile order: blockIdx % 8 is the XCD; consecutive tiles (same X panel) go to one XCD
     const int total = n_tiles * m_tiles;
     const int per_xcd = (total + 7) >> 3;
@@ -424,11 +458,11 @@ __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict_
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // consumer waves 2 (M) x 2 (N): the left column owns 6 column tiles (96 wide), the right one 5 (80)
     if (wave >= 4)
-        gemm_producer(smem, W, Xh, K, N, M, m0, n0);
+        gemm_producer(smem, W, K, N, n0);
     else if ((wave & 1) == 0)
-        gemm_consumer<6>(smem, Y, K, N, M, m0, n0, wave >> 1, 0);
+        gemm_consumer<6>(smem, Xh, Y, K, N, M, m0, n0, wave >> 1, 0);
     else
-        gemm_consumer<5>(smem, Y, K, N, M, m0, n0, wave >> 1, 96);
+        gemm_consumer<5>(smem, Xh, Y, K, N, M, m0, n0, wave >> 1, 96);
 }
 
 }  // namespace
@@ -442,9 +476,11 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
     GH_REQUIRE(ctx, gh_aligned(W, 2) && gh_aligned(X, 16) && gh_aligned(Y, 4), GALOIS_HIP_E_ALIGN,
                "mul_mat_q4_0_f32: W 2-byte, X 16-byte, Y 4-byte aligned");
     GH_BIND(ctx);
-    if (K % 256 == 0 && gh_aligned(W, 16)) {
-        // fp16 copy of X in the context's workspace (grown on demand, kept until the context dies)
-        const size_t need = (size_t)M * K * sizeof(_Float16);
+    if (K % 256 == 0 && gh_aligned(W, 16) && ((int64_t)M + 16) * K * 2 < ((int64_t)1 << 32)) {
+        // fp16 copy of X, tiled for the A fragments, in the context's workspace (grown on demand, kept
+        // until the context dies)
+        const int64_t m_pad = ((int64_t)M + 15) / 16 * 16;
+        const size_t need = (size_t)m_pad * K * sizeof(_Float16);
         if (ctx->ws_bytes < need) {
             GH_NOT_CAPTURING(ctx, "mul_mat_q4_0_f32: growing the fp16 workspace");
             hipError_t e = hipStreamSynchronize(ctx->stream);
@@ -457,8 +493,9 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
             ctx->ws_bytes = need;
         }
         _Float16 *Xh = (_Float16 *)ctx->ws;
-        const int64_t n8 = (int64_t)M * K / 8;
-        hipLaunchKernelGGL(f32_to_f16_rows, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, ctx->stream, X, Xh, n8);
+        const int64_t nchunks = m_pad * K / 8;
+        hipLaunchKernelGGL(f32_to_f16_tiles, dim3((unsigned)((nchunks + 255) / 256)), dim3(256), 0, ctx->stream, X, Xh, M,
+                           K, nchunks);
         const int n_tiles = (N + GN - 1) / GN, m_tiles = (M + GM - 1) / GM;
         const int total = n_tiles * m_tiles;
         const int grid = ((total + 7) / 8) * 8;
