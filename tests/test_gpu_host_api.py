@@ -95,8 +95,9 @@ def test_errors_instead_of_panics(gpu):
     with pytest.raises(g.GError) as e:   # the reference's (Cpu, Gpu, ..) arm is todo!()
         g.galois_matmul(g.Tensor.from_raw(w, [128, 1], g.Q4_0, cpu), x, y)
     assert e.value.kind == "Unimplemented"
-    with pytest.raises(g.GError) as e:   # f32 x f32 is todo!() in the reference too (src/cuda.rs:867-879)
-        g.galois_matmul(x, x, y)
+    g.galois_matmul(x, x, y)             # f32 x f32 (todo!() in the reference, src/cuda.rs:867-879) is served here
+    with pytest.raises(g.GError) as e:   # an i32 operand has no matmul arm (CudaMap2::map, src/cuda.rs:476-521)
+        g.galois_matmul(g.Tensor.zeros([128, 1], g.I32, gpu), x, y)
     assert e.value.kind == "Unimplemented"
     with pytest.raises(g.GError) as e:   # assert!(ne0 == ne01) in the reference (src/op.rs:1422)
         g.galois_matmul(a, x, g.Tensor.zeros([2, 1], g.F32, gpu))
