@@ -168,6 +168,23 @@ class Device:
         self._check(self._lib.galois_hip_dequantize_mul_mat_vec_q4_0(self._ctx, _ptr(vx), _ptr(y), _ptr(dst),
                                                                      ncols, nrows))
 
+    @staticmethod
+    def gemv_items(items):
+        """galois_hip_gemv_item array from dicts with vx, y, dst, ncols, nrows and optionally vx_up,
+        norm_weight, norm_eps, residual (build it once when the same launch is repeated)."""
+        arr = (_abi.GemvItem * max(1, len(items)))()
+        for a, it in zip(arr, items):
+            a.vx, a.y, a.dst = _ptr(it["vx"]), _ptr(it["y"]), _ptr(it["dst"])
+            a.vx_up, a.norm_weight = _ptr(it.get("vx_up")), _ptr(it.get("norm_weight"))
+            a.residual = _ptr(it.get("residual"))
+            a.ncols, a.nrows, a.norm_eps = it["ncols"], it["nrows"], it.get("norm_eps", 0.0)
+        arr.n_items = len(items)
+        return arr
+
+    def dequantize_mul_mat_vec_q4_0_group(self, items):
+        arr = items if isinstance(items, C.Array) else self.gemv_items(items)
+        self._check(self._lib.galois_hip_dequantize_mul_mat_vec_q4_0_group(self._ctx, arr, arr.n_items))
+
     def mul_mat_q4_0_f32(self, W, X, Y, K, N, M):
         self._check(self._lib.galois_hip_mul_mat_q4_0_f32(self._ctx, _ptr(W), _ptr(X), _ptr(Y), K, N, M))
 

@@ -12,6 +12,14 @@ i32 = C.c_int32
 f32 = C.c_float
 sz = C.c_size_t
 
+
+
+class GemvItem(C.Structure):
+    """galois_hip_gemv_item of include/galois_hip.h, field for field."""
+    _fields_ = [("vx", vp), ("vx_up", vp), ("y", vp), ("norm_weight", vp), ("residual", vp), ("dst", vp),
+                ("ncols", i32), ("nrows", i32), ("norm_eps", f32)]
+
+
 # name -> (restype, argtypes); must list every function the header declares
 PROTOTYPES = {
     "galois_hip_create": (i32, [i32, C.POINTER(c_ctx)]),
@@ -39,6 +47,7 @@ PROTOTYPES = {
     "galois_hip_quantize_row_q4_0": (i32, [c_ctx, vp, vp, C.c_int64]),
     "galois_hip_dequantize_row_q4_0": (i32, [c_ctx, vp, vp, C.c_int64]),
     "galois_hip_dequantize_mul_mat_vec_q4_0": (i32, [c_ctx, vp, vp, vp, i32, i32]),
+    "galois_hip_dequantize_mul_mat_vec_q4_0_group": (i32, [c_ctx, C.POINTER(GemvItem), i32]),
     "galois_hip_mul_mat_q4_0_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32]),
     "galois_hip_rms_norm_f32": (i32, [c_ctx, vp, vp, i32, i32, f32]),
     "galois_hip_rms_norm_mul_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, f32]),

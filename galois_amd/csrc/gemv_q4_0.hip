@@ -302,6 +302,217 @@ __global__ __launch_bounds__(256) void gemv_q4_0_generic(const uint16_t *__restr
     if (lane == 0) y[row] = acc;
 }
 
+// ---------------------------------------------------------------------------------------
+// Group kernel: up to GG_MAX matrix-vector products in one launch.
+//
+// A launch costs about as much as streaming 15-20 MB of weights.  Here the grids of several
+// products are laid end to end: a workgroup finds its matrix from its block index and then
+// does what a workgroup of gemv_q4_0_dot8 does (single pass, K <= 12288); the hardware hands
+// workgroups to CUs as they free up, which balances matrices of different shapes.
+//
+// Fused around the product, so that a decode step needs no separate launches for them:
+//   - RMSNorm (+ weight) of the activation vector while it is prepared (rms_norm.cu:13-49
+//     followed by mul.cu:3-12): every workgroup reads the whole vector anyway;
+//   - a residual added to the result (add.cu:3-12);
+//   - a second matrix on the same activations whose result is multiplied with silu of the
+//     first's (unary.cu:1-10 then mul.cu:3-12): the SwiGLU gate / up pair.
+constexpr int GG_MAX = 8;
+constexpr int GG_MAX_SLOTS = kChunkSlots;  // K <= 12288: one LDS pass
+
+struct gg_item {
+    const uint8_t *W;
+    const uint8_t *W2;      // up matrix of a SwiGLU pair, or null
+    float *dst;
+    const float *residual;  // or null
+    const float *x;
+    const float *norm_w;    // RMSNorm weight or null
+    float eps;
+    int32_t N;
+    int32_t nslots;
+    int32_t pad;
+};
+struct gg_args {
+    int32_t blk0[GG_MAX];  // first block of each matrix; unused entries hold INT_MAX
+    gg_item item[GG_MAX];
+};
+
+// A wave owns R slots per lane: R rows, or R / 2 rows of a gate / up pair; a workgroup WAVES times that.
+// PG: activation groups (8 values) one thread prepares at most; NORM: the vector is normalised first.
+template <int L, int R, int WAVES, int PG, int OCC, bool NORM>
+__global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args a) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    __shared__ float red[WAVES];
+    constexpr int SD = slot_lds<L>::dwords;
+    constexpr int THREADS = WAVES * 64;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    GH_TSTAMP(0);
+
+    int ii = 0;
+#pragma unroll
+    for (int k = 1; k < GG_MAX; k++)
+        if ((int)blockIdx.x >= a.blk0[k]) ii = k;
+    const gg_item &it = a.item[ii];
+    const uint8_t *const W = it.W, *const W2 = it.W2;
+    const bool dual = W2 != nullptr;
+    const int N = it.N, ns = it.nslots;
+    const int rw = dual ? R / 2 : R;  // rows per wave
+    const int row0 = (((int)blockIdx.x - a.blk0[ii]) * WAVES + wave) * rw;
+    const size_t row_bytes = (size_t)ns * sizeof(q4_slot);
+    GH_TSTAMP(1);
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+
+    // ---- activation preparation: task = (slot, weight-dword group).  Loads retire in order, so the activations
+    // are requested first and the first weights right behind them: the preparation then runs while the weights
+    // are in flight.
+    q4_slot q0[R];
+    {
+        const float *xg = it.x, *wg = it.norm_w;
+        float2 v[PG][4], nw[NORM ? PG : 1][4];
+#pragma unroll
+        for (int p = 0; p < PG; p++) {
+            const int idx = threadIdx.x + p * THREADS;
+            if (idx < ns * 8) {
+                const int slot = idx >> 3, g = idx & 7;
+#pragma unroll
+                for (int t = 0; t < 4; t += 2) {
+                    const int b = slot * 64 + xprep::group_x_index(g, 2 * t);  // even by construction
+                    v[p][t] = *reinterpret_cast<const float2 *>(xg + b);
+                    v[p][t + 1] = *reinterpret_cast<const float2 *>(xg + b + 16);
+                    if (NORM) {
+                        nw[NORM ? p : 0][t] = *reinterpret_cast<const float2 *>(wg + b);
+                        nw[NORM ? p : 0][t + 1] = *reinterpret_cast<const float2 *>(wg + b + 16);
+                    }
+                }
+            }
+        }
+        // q[j] = slot `lane` of row row0 + j of W; for a gate / up pair q[j] = row row0 + j of W (j < R/2) or of W2.
+        // Rows past N are loaded from row N - 1 and never stored.
+        {
+            const int s = min(lane, ns - 1);
+#pragma unroll
+            for (int j = 0; j < R; j++) {
+                const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
+                const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
+                load_slot(q0[j], base + (size_t)row * row_bytes + (size_t)s * sizeof(q4_slot));
+            }
+        }
+        GH_TSTAMP(2);
+        if (NORM) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int p = 0; p < PG; p++)
+                if (threadIdx.x + p * THREADS < ns * 8) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) ss += v[p][t].x * v[p][t].x + v[p][t].y * v[p][t].y;
+                }
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WAVES; w++) tot += red[w];
+            const float inv = rsqrtf(tot / (float)(ns * 64) + it.eps);
+#pragma unroll
+            for (int p = 0; p < PG; p++)
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    v[p][t].x = (inv * v[p][t].x) * nw[NORM ? p : 0][t].x;
+                    v[p][t].y = (inv * v[p][t].y) * nw[NORM ? p : 0][t].y;
+                }
+        }
+#pragma unroll
+        for (int p = 0; p < PG; p++) {
+            const int idx = threadIdx.x + p * THREADS;
+            if (idx < ns * 8) {
+                const int slot = idx >> 3, g = idx & 7;
+                const float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
+                                     v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
+                uint32_t amax = 0;
+#pragma unroll
+                for (int j = 0; j < 8; j++) amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
+                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0xB1, 0xF, 0xF, true));
+                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0x4E, 0xF, 0xF, true));
+                float mult, scale;
+                xprep::block_scales<L>(amax, &mult, &scale);
+                uint32_t planes[L];
+                xprep::make_planes<L>(x8, mult, planes);
+                uint32_t *dst = lds + slot * SD;
+#pragma unroll
+                for (int l = 0; l < L; l++) dst[l * 8 + g] = planes[l];
+                if ((g & 3) == 0) dst[8 * L + (g >> 2)] = __builtin_bit_cast(uint32_t, scale);
+            }
+        }
+    }
+    GH_TSTAMP(3);
+    __syncthreads();
+    GH_TSTAMP(4);
+
+    for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
+        const bool act = sl < ns;
+        const int s_ld = min(sl, ns - 1);
+        uint32_t xl[L][8];
+        float sA, sB;
+        {
+            const uint32_t *src = lds + s_ld * SD;
+#pragma unroll
+            for (int l = 0; l < L; l++) {
+                const uint4 lo4 = *reinterpret_cast<const uint4 *>(src + l * 8);
+                const uint4 hi4 = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
+                xl[l][0] = lo4.x, xl[l][1] = lo4.y, xl[l][2] = lo4.z, xl[l][3] = lo4.w;
+                xl[l][4] = hi4.x, xl[l][5] = hi4.y, xl[l][6] = hi4.z, xl[l][7] = hi4.w;
+            }
+            const uint2 sc = *reinterpret_cast<const uint2 *>(src + 8 * L);
+            sA = __builtin_bit_cast(float, sc.x);
+            sB = __builtin_bit_cast(float, sc.y);
+        }
+        q4_slot q[R];
+        if (sl == lane) {
+#pragma unroll
+            for (int j = 0; j < R; j++) q[j] = q0[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < R; j++) {
+                const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
+                const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
+                load_slot(q[j], base + (size_t)row * row_bytes + (size_t)s_ld * sizeof(q4_slot));
+            }
+        }
+        if (act) {
+#pragma unroll
+            for (int j = 0; j < R; j++) acc[j] += slot_dot<L>(q[j], xl, sA, sB);
+        }
+    }
+    GH_TSTAMP(5);
+
+    // every total lands in lane 63; lane j picks up row j so the wave stores its rows at once
+    float out = 0.0f;
+    if (dual) {
+#pragma unroll
+        for (int j = 0; j < R / 2; j++) {
+            float g = wave_sum_to_lane63(acc[j]), up = wave_sum_to_lane63(acc[R / 2 + j]);
+            g = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, g), 63));
+            up = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, up), 63));
+            if (lane == j) out = g / (1.0f + expf(-g)) * up;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            float t = wave_sum_to_lane63(acc[j]);
+            t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
+            if (lane == j) out = t;
+        }
+    }
+    if (lane < rw && row0 + lane < N) {
+        if (it.residual) out += it.residual[row0 + lane];
+        it.dst[row0 + lane] = out;
+    }
+    GH_TSTAMP(6);
+}
+
 template <int L, int R, int G, int WAVES, int OCC>
 void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst, int nslots, int N) {
     const int rows_per_wg = WAVES * R * G;
@@ -322,6 +533,75 @@ void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst
                            dst, nslots, N);
 }
 
+// Host side of the group kernel: checks, the block range of every matrix, launch.
+template <int L, int R, int WAVES, int OCC>
+void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, int max_slots, bool norm) {
+    const dim3 grid(blocks), block(WAVES * 64);
+    const size_t lds = (size_t)max_slots * slot_lds<L>::dwords * sizeof(uint32_t);
+    constexpr int PGMAX = (kChunkSlots * 8 + WAVES * 64 - 1) / (WAVES * 64);
+    constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
+    if (max_slots <= 64) {
+        if (norm)
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true>), grid, block, lds, ctx->stream, a);
+        else
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, false>), grid, block, lds, ctx->stream, a);
+    } else {
+        if (norm)
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, true>), grid, block, lds, ctx->stream, a);
+        else
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, false>), grid, block, lds, ctx->stream, a);
+    }
+}
+
+int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what) {
+    GH_REQUIRE(ctx, items != nullptr, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, n_items >= 1 && n_items <= GG_MAX, GALOIS_HIP_E_SHAPE, "gemv group: 1 to 8 products per call");
+    gg_args a;
+    memset(&a, 0, sizeof(a));
+    int32_t max_slots = 0;
+    int64_t rows = 0;
+    bool norm = false;
+    for (int i = 0; i < GG_MAX; i++) a.blk0[i] = 0x7FFFFFFF;
+    for (int i = 0; i < n_items; i++) {
+        const galois_hip_gemv_item &s = items[i];
+        GH_REQUIRE(ctx, s.vx && s.y && s.dst, GALOIS_HIP_E_NULL, what);
+        GH_REQUIRE(ctx, s.ncols > 0 && s.nrows > 0 && s.ncols % 64 == 0 && s.ncols / 64 <= GG_MAX_SLOTS, GALOIS_HIP_E_SHAPE,
+                   "gemv group: ncols must be a positive multiple of 64, at most 12288; nrows positive");
+        GH_REQUIRE(ctx, gh_aligned(s.vx, 4) && gh_aligned(s.vx_up, 4) && gh_aligned(s.y, 8) && gh_aligned(s.norm_weight, 8) &&
+                            gh_aligned(s.residual, 4) && gh_aligned(s.dst, 4),
+                   GALOIS_HIP_E_ALIGN, "gemv group: matrices 4-byte, activations and norm weights 8-byte, vectors 4-byte aligned");
+        if (i == 0) norm = s.norm_weight != nullptr;
+        GH_REQUIRE(ctx, (s.norm_weight != nullptr) == norm, GALOIS_HIP_E_UNSUPPORTED,
+                   "gemv group: either every product of a call normalises its activations or none does");
+        gg_item &d = a.item[i];
+        d.W = (const uint8_t *)s.vx, d.W2 = (const uint8_t *)s.vx_up, d.dst = s.dst, d.residual = s.residual;
+        d.x = s.y, d.norm_w = s.norm_weight, d.eps = s.norm_eps, d.N = s.nrows, d.nslots = s.ncols / 64;
+        if (d.nslots > max_slots) max_slots = d.nslots;
+        rows += (int64_t)s.nrows * (s.vx_up ? 2 : 1);
+    }
+    // Workgroup shape by rows per CU, as for the one-product kernel: few rows -> 16 waves x 1 slot so every SIMD has
+    // work; more rows -> 8 waves x 2 slots, four workgroups resident per CU.  A gate / up pair needs 2 slots per lane.
+    bool any_dual = false;
+    for (int i = 0; i < n_items; i++) any_dual |= items[i].vx_up != nullptr;
+    int cfg = ctx->gemv_config;
+    if (cfg != 1 && cfg != 4) cfg = (!any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16) ? 1 : 4;
+    if (any_dual) cfg = 4;
+    const int slots_per_wg = cfg == 1 ? 16 : 16;  // WAVES * R of the two shapes
+    int64_t blocks = 0;
+    for (int i = 0; i < n_items; i++) {
+        const int64_t rows_per_wg = items[i].vx_up ? slots_per_wg / 2 : slots_per_wg;
+        a.blk0[i] = (int32_t)blocks;
+        blocks += (items[i].nrows + rows_per_wg - 1) / rows_per_wg;
+        GH_REQUIRE(ctx, blocks < 0x7FFFFFFF, GALOIS_HIP_E_SHAPE, "gemv group: too many rows");
+    }
+    GH_BIND(ctx);
+    if (cfg == 1)
+        launch_group_cfg<5, 1, 16, 4>(ctx, a, (unsigned)blocks, max_slots, norm);
+    else
+        launch_group_cfg<5, 2, 8, 4>(ctx, a, (unsigned)blocks, max_slots, norm);
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
 }  // namespace
 
 extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, const void *vx, const float *y,
@@ -340,6 +620,12 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, c
         // activation preparation is spread over 1024 threads; more rows -> 8 waves x 2 rows, several
         // workgroups resident per CU so one's preparation overlaps another's streaming.
         int cfg = ctx->gemv_config;
+        if (cfg == 6 && ncols <= 64 * GG_MAX_SLOTS) {
+            galois_hip_gemv_item it;
+            memset(&it, 0, sizeof(it));
+            it.vx = vx, it.y = y, it.dst = dst, it.ncols = ncols, it.nrows = nrows;
+            return launch_group(ctx, &it, 1, "dequantize_mul_mat_vec_q4_0");
+        }
         if (cfg == 0) {
             const int64_t rows_per_cu = ((int64_t)nrows + ctx->n_cu - 1) / ctx->n_cu;
             cfg = rows_per_cu <= 16 ? 1 : 4;
@@ -357,4 +643,10 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, c
                            y, dst, ncols / 32, nrows);
     }
     GH_LAUNCH_CHECK(ctx, "dequantize_mul_mat_vec_q4_0 launch");
+}
+
+extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items,
+                                                                int32_t n_items) {
+    GH_REQUIRE_CTX(ctx);
+    return launch_group(ctx, items, n_items, "dequantize_mul_mat_vec_q4_0_group");
 }

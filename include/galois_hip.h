@@ -118,6 +118,34 @@ int32_t galois_hip_dequantize_row_q4_0(galois_hip_ctx *ctx, const void *x, float
 int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, const void *vx, const float *y,
                                                float *dst, int32_t ncols, int32_t nrows);
 
+/* Several decode GEMVs in one launch.  The reference launches one kernel per product and per
+ * batch slice (the loop at src/cuda.rs:1026-1034) and one more for every op around it; on this
+ * device a launch costs as much as streaming 15-20 MB of weights, so the products of a decode
+ * step that do not depend on each other (q | k | v, gate | up) go out together and the row ops
+ * next to them ride along:
+ *   norm_weight != NULL: y is replaced by rms_norm(y, norm_eps) * norm_weight before the product
+ *     (rms_norm_f32 + mul_f32, src/cuda.rs:1146-1215);
+ *   vx_up != NULL: dst = silu(vx . y) * (vx_up . y), the SwiGLU pair (silu_f32 then mul_f32,
+ *     src/cuda.rs:1665-1688, 1190-1215); vx_up has the shape of vx;
+ *   residual != NULL: residual[row] is added to the result (add_f32, src/cuda.rs:1188-1244);
+ *     residual may be dst.
+ * Each product is what galois_hip_dequantize_mul_mat_vec_q4_0 computes.  1 <= n_items <= 8;
+ * ncols % 64 == 0 and ncols <= 12288; matrices 4-byte aligned, y and norm_weight 8-byte aligned;
+ * either every product of a call has a norm_weight or none has.  The items array is read during
+ * the call only. */
+typedef struct galois_hip_gemv_item {
+    const void *vx;
+    const void *vx_up;
+    const float *y;
+    const float *norm_weight;
+    const float *residual;
+    float *dst;
+    int32_t ncols, nrows;
+    float norm_eps;
+} galois_hip_gemv_item;
+int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items,
+                                                     int32_t n_items);
+
 /* Prefill matmul.  Replaces quantize_q8_1 + mul_mat_q4_0 (src/cuda.rs:1035-1136 ->
  * matmul.cu:133-174,452-504) with one call: Y[m*N + n] = sum_k deq(W)[n,k] * X[m*K + k]
  * (output layout of matmul.cu:359).  W tiles are dequantised to fp16 in LDS, X is
