@@ -329,7 +329,7 @@ struct gg_item {
     float eps;
     int32_t N;
     int32_t nslots;
-    int32_t pad;
+    int32_t groups;  // row groups a wave works through, one after the other: amortises the preparation when N is large
 };
 struct gg_args {
     int32_t blk0[GG_MAX];  // first block of each matrix; unused entries hold INT_MAX
@@ -356,8 +356,11 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     const uint8_t *const W = it.W, *const W2 = it.W2;
     const bool dual = W2 != nullptr;
     const int N = it.N, ns = it.nslots;
-    const int rw = dual ? R / 2 : R;  // rows per wave
-    const int row0 = (((int)blockIdx.x - a.blk0[ii]) * WAVES + wave) * rw;
+    const int rw = dual ? R / 2 : R;  // rows per wave and group
+    const int groups = it.groups;
+    // group g of the workgroup's waves covers WAVES * rw consecutive rows: neighbouring waves read neighbouring rows
+    const int wg_row0 = ((int)blockIdx.x - a.blk0[ii]) * (WAVES * rw * groups);
+    int row0 = wg_row0 + wave * rw;
     const size_t row_bytes = (size_t)ns * sizeof(q4_slot);
     GH_TSTAMP(1);
 
@@ -451,64 +454,68 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     __syncthreads();
     GH_TSTAMP(4);
 
-    for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
-        const bool act = sl < ns;
-        const int s_ld = min(sl, ns - 1);
-        uint32_t xl[L][8];
-        float sA, sB;
-        {
-            const uint32_t *src = lds + s_ld * SD;
+    for (int g = 0; g < groups; g++, row0 += WAVES * rw) {
+        if (g > 0 && row0 >= N) break;  // wave-uniform
+        for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
+            const bool act = sl < ns;
+            const int s_ld = min(sl, ns - 1);
+            uint32_t xl[L][8];
+            float sA, sB;
+            {
+                const uint32_t *src = lds + s_ld * SD;
 #pragma unroll
-            for (int l = 0; l < L; l++) {
-                const uint4 lo4 = *reinterpret_cast<const uint4 *>(src + l * 8);
-                const uint4 hi4 = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
-                xl[l][0] = lo4.x, xl[l][1] = lo4.y, xl[l][2] = lo4.z, xl[l][3] = lo4.w;
-                xl[l][4] = hi4.x, xl[l][5] = hi4.y, xl[l][6] = hi4.z, xl[l][7] = hi4.w;
+                for (int l = 0; l < L; l++) {
+                    const uint4 lo4 = *reinterpret_cast<const uint4 *>(src + l * 8);
+                    const uint4 hi4 = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
+                    xl[l][0] = lo4.x, xl[l][1] = lo4.y, xl[l][2] = lo4.z, xl[l][3] = lo4.w;
+                    xl[l][4] = hi4.x, xl[l][5] = hi4.y, xl[l][6] = hi4.z, xl[l][7] = hi4.w;
+                }
+                const uint2 sc = *reinterpret_cast<const uint2 *>(src + 8 * L);
+                sA = __builtin_bit_cast(float, sc.x);
+                sB = __builtin_bit_cast(float, sc.y);
             }
-            const uint2 sc = *reinterpret_cast<const uint2 *>(src + 8 * L);
-            sA = __builtin_bit_cast(float, sc.x);
-            sB = __builtin_bit_cast(float, sc.y);
-        }
-        q4_slot q[R];
-        if (sl == lane) {
+            q4_slot q[R];
+            if (g == 0 && sl == lane) {
 #pragma unroll
-            for (int j = 0; j < R; j++) q[j] = q0[j];
+                for (int j = 0; j < R; j++) q[j] = q0[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < R; j++) {
+                    const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
+                    const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
+                    load_slot(q[j], base + (size_t)row * row_bytes + (size_t)s_ld * sizeof(q4_slot));
+                }
+            }
+            if (act) {
+#pragma unroll
+                for (int j = 0; j < R; j++) acc[j] += slot_dot<L>(q[j], xl, sA, sB);
+            }
+        }
+
+        // every total lands in lane 63; lane j picks up row j so the wave stores its rows at once
+        float out = 0.0f;
+        if (dual) {
+#pragma unroll
+            for (int j = 0; j < R / 2; j++) {
+                float gt = wave_sum_to_lane63(acc[j]), up = wave_sum_to_lane63(acc[R / 2 + j]);
+                gt = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gt), 63));
+                up = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, up), 63));
+                if (lane == j) out = gt / (1.0f + expf(-gt)) * up;
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < R; j++) {
-                const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
-                const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
-                load_slot(q[j], base + (size_t)row * row_bytes + (size_t)s_ld * sizeof(q4_slot));
+                float t = wave_sum_to_lane63(acc[j]);
+                t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
+                if (lane == j) out = t;
             }
         }
-        if (act) {
-#pragma unroll
-            for (int j = 0; j < R; j++) acc[j] += slot_dot<L>(q[j], xl, sA, sB);
+        if (lane < rw && row0 + lane < N) {
+            if (it.residual) out += it.residual[row0 + lane];
+            it.dst[row0 + lane] = out;
         }
-    }
-    GH_TSTAMP(5);
-
-    // every total lands in lane 63; lane j picks up row j so the wave stores its rows at once
-    float out = 0.0f;
-    if (dual) {
 #pragma unroll
-        for (int j = 0; j < R / 2; j++) {
-            float g = wave_sum_to_lane63(acc[j]), up = wave_sum_to_lane63(acc[R / 2 + j]);
-            g = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, g), 63));
-            up = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, up), 63));
-            if (lane == j) out = g / (1.0f + expf(-g)) * up;
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < R; j++) {
-            float t = wave_sum_to_lane63(acc[j]);
-            t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
-            if (lane == j) out = t;
-        }
-    }
-    if (lane < rw && row0 + lane < N) {
-        if (it.residual) out += it.residual[row0 + lane];
-        it.dst[row0 + lane] = out;
+        for (int j = 0; j < R; j++) acc[j] = 0.0f;
     }
     GH_TSTAMP(6);
 }
@@ -586,10 +593,16 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     int cfg = ctx->gemv_config;
     if (cfg != 1 && cfg != 4) cfg = (!any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16) ? 1 : 4;
     if (any_dual) cfg = 4;
-    const int slots_per_wg = cfg == 1 ? 16 : 16;  // WAVES * R of the two shapes
+    const int slots_per_wg = 16;  // WAVES * R of both shapes
     int64_t blocks = 0;
     for (int i = 0; i < n_items; i++) {
-        const int64_t rows_per_wg = items[i].vx_up ? slots_per_wg / 2 : slots_per_wg;
+        // more rows per workgroup when there are plenty: the preparation is paid once per workgroup
+        const int64_t wgs1 = ((int64_t)items[i].nrows * (items[i].vx_up ? 2 : 1) + slots_per_wg - 1) / slots_per_wg;
+        int groups = ctx->gemv_units_per_wave;
+        if (groups <= 0) groups = wgs1 >= 4 * (int64_t)ctx->n_cu ? 2 : 1;  // measured: 9 % on the 32000-row matrix
+        groups = groups < 1 ? 1 : (groups > 4 ? 4 : groups);
+        a.item[i].groups = groups;
+        const int64_t rows_per_wg = (items[i].vx_up ? slots_per_wg / 2 : slots_per_wg) * groups;
         a.blk0[i] = (int32_t)blocks;
         blocks += (items[i].nrows + rows_per_wg - 1) / rows_per_wg;
         GH_REQUIRE(ctx, blocks < 0x7FFFFFFF, GALOIS_HIP_E_SHAPE, "gemv group: too many rows");
@@ -620,7 +633,8 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, c
         // activation preparation is spread over 1024 threads; more rows -> 8 waves x 2 rows, several
         // workgroups resident per CU so one's preparation overlaps another's streaming.
         int cfg = ctx->gemv_config;
-        if (cfg == 6 && ncols <= 64 * GG_MAX_SLOTS) {
+        // many rows: the group kernel's two row groups per wave halve the preparation per row
+        if ((cfg == 6 || (cfg == 0 && nrows >= 64 * ctx->n_cu)) && ncols <= 64 * GG_MAX_SLOTS) {
             galois_hip_gemv_item it;
             memset(&it, 0, sizeof(it));
             it.vx = vx, it.y = y, it.dst = dst, it.ncols = ncols, it.nrows = nrows;

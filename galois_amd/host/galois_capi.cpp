@@ -161,11 +161,11 @@ void *galois_host_llama_tensor(void *m, const char *name, int layer) {
 void *galois_host_llama_logits(void *m) { return (void *)&((LlamaDecoder *)m)->logits(); }
 size_t galois_host_llama_ops_per_step(void *m) { return ((LlamaDecoder *)m)->ops_per_step(); }
 int galois_host_llama_decode(void *m, int32_t token, int32_t n_past, int fused) {
-    GResult r = ((LlamaDecoder *)m)->decode(token, n_past, fused != 0);
+    GResult r = ((LlamaDecoder *)m)->decode(token, n_past, fused);
     return r.ok() ? 0 : fail(r);
 }
 int galois_host_llama_capture(void *m, int32_t token, int32_t n_past, int fused) {
-    GResult r = ((LlamaDecoder *)m)->capture(token, n_past, fused != 0);
+    GResult r = ((LlamaDecoder *)m)->capture(token, n_past, fused);
     return r.ok() ? 0 : fail(r);
 }
 int galois_host_llama_replay(void *m) {
@@ -196,7 +196,7 @@ int galois_host_llama_time_steps(void *m, void *dev, int32_t token, int32_t n_pa
     if (!st) st = galois_hip_event_create(ctx, &e1);
     if (!st) st = galois_hip_event_record(ctx, e0);
     GResult r;
-    for (int i = 0; i < n && !st && r.ok(); i++) r = ((LlamaDecoder *)m)->decode(token, n_past, fused != 0);
+    for (int i = 0; i < n && !st && r.ok(); i++) r = ((LlamaDecoder *)m)->decode(token, n_past, fused);
     if (!st) st = galois_hip_event_record(ctx, e1);
     if (!st) st = galois_hip_event_elapsed_ms(ctx, e0, e1, ms);
     galois_hip_event_destroy(ctx, e0);

@@ -38,6 +38,37 @@ GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst) {
                                               (float *)dst.data(), (int64_t)gate.dim().elem_count()));
 }
 
+GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
+    if (items.empty() || items.size() > 8) return err(GError::ShapeError, "galois_matvec_group: 1 to 8 products");
+    galois_hip_gemv_item it[8];
+    std::shared_ptr<CudaDevice> dev;
+    for (size_t i = 0; i < items.size(); i++) {
+        const MatvecItem &m = items[i];
+        if (!m.w || !m.x || !m.dst) return err(GError::Unexpected, "galois_matvec_group: w, x and dst are required");
+        for (const Tensor *t : {m.w, m.w_up, m.x, m.norm_weight, m.residual, (const Tensor *)m.dst}) {
+            if (!t) continue;
+            if (!t->device().is_gpu()) return err(GError::Unimplemented, "galois_matvec_group: Gpu tensors only");
+            if (!dev) dev = t->device().gpu;
+            if (t->device().gpu != dev) return err(GError::Unimplemented, "galois_matvec_group: one device");
+            if (!t->dim().ggml_is_contiguous(t->dtype())) return err(GError::Unimplemented, "galois_matvec_group: contiguous tensors only");
+        }
+        if (m.w->dtype() != GGmlType::Q4_0 || (m.w_up && m.w_up->dtype() != GGmlType::Q4_0))
+            return err(GError::Unimplemented, "galois_matvec_group: Q4_0 matrices only");
+        for (const Tensor *t : {m.x, m.norm_weight, m.residual, (const Tensor *)m.dst})
+            if (t && t->dtype() != GGmlType::F32) return err(GError::Unimplemented, "galois_matvec_group: F32 vectors only");
+        const size_t K = m.w->dim().shape[0], N = m.w->dim().shape[1];
+        if (m.w->dim().elem_count() != K * N || m.x->dim().elem_count() != K || m.dst->dim().elem_count() != N ||
+            (m.w_up && (m.w_up->dim().shape[0] != K || m.w_up->dim().elem_count() != K * N)) ||
+            (m.norm_weight && m.norm_weight->dim().elem_count() != K) || (m.residual && m.residual->dim().elem_count() != N))
+            return err(GError::ShapeError, "galois_matvec_group: w [K, N], w_up [K, N], x and norm_weight K, dst and residual N elements");
+        it[i].vx = m.w->data(), it[i].vx_up = m.w_up ? m.w_up->data() : nullptr, it[i].y = (const float *)m.x->data();
+        it[i].norm_weight = m.norm_weight ? (const float *)m.norm_weight->data() : nullptr;
+        it[i].residual = m.residual ? (const float *)m.residual->data() : nullptr;
+        it[i].dst = (float *)m.dst->data(), it[i].ncols = (int32_t)K, it[i].nrows = (int32_t)N, it[i].norm_eps = m.eps;
+    }
+    return dev->check(galois_hip_dequantize_mul_mat_vec_q4_0_group(dev->ctx(), it, (int32_t)items.size()));
+}
+
 static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t ne1 = 0, size_t ne2 = 0) {
     const size_t shape[3] = {ne0, ne1, ne2};
     return Tensor::zeros(ne2 ? 3 : (ne1 ? 2 : 1), shape, ty, dev, t);
@@ -118,7 +149,7 @@ GResult LlamaDecoder::set_inputs(int32_t token, int32_t n_past) {
 
 // The op sequence of one token.  Shapes in ggml order [ne0, ne1, ne2]; L = n_past + 1 keys are visible,
 // so the softmax needs no mask.
-GResult LlamaDecoder::step(int32_t n_past, bool fused) {
+GResult LlamaDecoder::step(int32_t n_past, int fused) {
     const size_t E = hp_.n_embd, H = hp_.n_head, D = E / H, L = (size_t)n_past + 1, C = hp_.n_ctx;
     RopeCustomOption rope;
     rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;
@@ -142,11 +173,23 @@ GResult LlamaDecoder::step(int32_t n_past, bool fused) {
         G_TRY(qr_.view(0, 3, qs, &q3));
     }
     G_TRY(galois_get_rows(tok_embd_, tok_id_, x_)); ops++;
+    const bool grouped = fused >= 2;
+    auto item = [&](const Tensor &w, const Tensor &x, Tensor &dst) {
+        MatvecItem m;
+        m.w = &w, m.x = &x, m.dst = &dst, m.eps = hp_.rms_eps;
+        return m;
+    };
     for (Layer &l : layers_) {
-        G_TRY(norm(x_, l.attn_norm, a_));
-        G_TRY(galois_matmul(l.wq, a_, q_));
-        G_TRY(galois_matmul(l.wk, a_, k_));
-        G_TRY(galois_matmul(l.wv, a_, v_)); ops += 3;
+        if (grouped) {  // rms_norm * weight + the three projections: one launch
+            MatvecItem mq = item(l.wq, x_, q_), mk_ = item(l.wk, x_, k_), mv = item(l.wv, x_, v_);
+            mq.norm_weight = mk_.norm_weight = mv.norm_weight = &l.attn_norm;
+            G_TRY(galois_matvec_group({mq, mk_, mv})); ops++;
+        } else {
+            G_TRY(norm(x_, l.attn_norm, a_));
+            G_TRY(galois_matmul(l.wq, a_, q_));
+            G_TRY(galois_matmul(l.wk, a_, k_));
+            G_TRY(galois_matmul(l.wv, a_, v_)); ops += 3;
+        }
         Tensor qv, kv;
         const size_t hs[3] = {D, H, 1};
         G_TRY(q_.view(0, 3, hs, &qv));
@@ -174,6 +217,18 @@ GResult LlamaDecoder::step(int32_t n_past, bool fused) {
         G_TRY(galois_matmul(vc, p, o_)); ops++;
         Tensor o_flat;
         G_TRY(o_.view(0, 2, row, &o_flat));
+        if (grouped) {
+            MatvecItem mo = item(l.wo, o_flat, x1_);  // x1 = wo . o + x
+            mo.residual = &x_;
+            G_TRY(galois_matvec_group({mo})); ops++;
+            MatvecItem mg = item(l.w_gate, x1_, h_);  // h = silu(w_gate . n) * (w_up . n), n = rms_norm(x1) * ffn_norm
+            mg.w_up = &l.w_up, mg.norm_weight = &l.ffn_norm;
+            G_TRY(galois_matvec_group({mg})); ops++;
+            MatvecItem md = item(l.w_down, h_, x_);   // x = w_down . h + x1
+            md.residual = &x1_;
+            G_TRY(galois_matvec_group({md})); ops++;
+            continue;
+        }
         G_TRY(galois_matmul(l.wo, o_flat, ao_));
         G_TRY(galois_add(ao_, x_, x1_)); ops += 2;
         G_TRY(norm(x1_, l.ffn_norm, f_));
@@ -188,18 +243,24 @@ GResult LlamaDecoder::step(int32_t n_past, bool fused) {
         G_TRY(galois_matmul(l.w_down, h_, d_));
         G_TRY(galois_add(d_, x1_, x_)); ops += 2;
     }
-    G_TRY(norm(x_, out_norm_, a_));
-    G_TRY(galois_matmul(output_, a_, logits_)); ops++;
+    if (grouped) {
+        MatvecItem ml = item(output_, x_, logits_);
+        ml.norm_weight = &out_norm_;
+        G_TRY(galois_matvec_group({ml})); ops++;
+    } else {
+        G_TRY(norm(x_, out_norm_, a_));
+        G_TRY(galois_matmul(output_, a_, logits_)); ops++;
+    }
     n_ops_ = ops;
     return GError{};
 }
 
-GResult LlamaDecoder::decode(int32_t token, int32_t n_past, bool fused) {
+GResult LlamaDecoder::decode(int32_t token, int32_t n_past, int fused) {
     G_TRY(set_inputs(token, n_past));
     return step(n_past, fused);
 }
 
-GResult LlamaDecoder::capture(int32_t token, int32_t n_past, bool fused) {
+GResult LlamaDecoder::capture(int32_t token, int32_t n_past, int fused) {
     galois_hip_ctx *ctx = dev_.gpu->ctx();
     if (graph_) {
         G_TRY(dev_.gpu->check(galois_hip_graph_destroy(ctx, graph_)));

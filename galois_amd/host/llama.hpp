@@ -34,9 +34,11 @@ class LlamaDecoder {
     // Enqueues one step for `token` at position n_past (attention over n_past + 1 keys); logits() holds the
     // result once the stream is synchronised (to_cpu_tensor does that).  fused = use the library's fused
     // rms_norm*weight and silu*up kernels instead of two ops each.
-    GResult decode(int32_t token, int32_t n_past, bool fused);
+    // fused = 2 additionally sends the Q4_0 matrix-vector products out in grouped launches (q | k | v together,
+    // gate | up as a SwiGLU pair) with the norms, silu * up and the residual adds riding along: 12 launches per layer.
+    GResult decode(int32_t token, int32_t n_past, int fused);
     // Records the same step as a graph / replays the recorded step.
-    GResult capture(int32_t token, int32_t n_past, bool fused);
+    GResult capture(int32_t token, int32_t n_past, int fused);
     GResult replay();
     const Tensor &logits() const { return logits_; }
     const LlamaHParams &hparams() const { return hp_; }
@@ -47,7 +49,7 @@ class LlamaDecoder {
         Tensor attn_norm, ffn_norm, wq, wk, wv, wo, w_gate, w_up, w_down, k_cache, v_cache;
     };
     GResult set_inputs(int32_t token, int32_t n_past);
-    GResult step(int32_t n_past, bool fused);
+    GResult step(int32_t n_past, int fused);
 
     LlamaHParams hp_;
     Device dev_;
@@ -64,5 +66,15 @@ class LlamaDecoder {
 // weight multiply, and silu(gate) * up, each as one kernel.
 GResult galois_rms_norm_mul(const Tensor &src, const Tensor &weight, Tensor &dst, float eps);
 GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst);
+
+// Several Q4_0 matrix-vector products in one launch (galois_hip_dequantize_mul_mat_vec_q4_0_group): per product
+// dst = w . x, where x is first replaced by rms_norm(x, eps) * norm_weight when norm_weight is set, the result
+// becomes silu(w . x) * (w_up . x) when w_up is set, and residual is added when set (it may be dst).
+struct MatvecItem {
+    const Tensor *w = nullptr, *w_up = nullptr, *x = nullptr, *norm_weight = nullptr, *residual = nullptr;
+    Tensor *dst = nullptr;
+    float eps = 0.0f;
+};
+GResult galois_matvec_group(const std::vector<MatvecItem> &items);
 
 }  // namespace galois

@@ -87,11 +87,12 @@ def test_decode_step_matches_oracle_with_a_filled_cache(gdev):
     dec = g.LlamaDecoder(gdev, **hp)
     _load(dec, w, kc, vc)
     ref = _ref_step(w, hp, kc.copy(), vc.copy(), 123, n_past)
-    for fused in (False, True):
+    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1)):
         _load(dec, w, kc, vc)
         dec.decode(123, n_past, fused)
         _check(dec.logits(), ref, 1e-4)
-    assert dec.ops_per_step() == 1 + hp["n_layer"] * 20 + 2      # fused: 20 launches per layer
+        # launches: embedding lookup + per layer + final norm and lm head (fused = 2: grouped products, 12 per layer)
+        assert dec.ops_per_step() == 1 + hp["n_layer"] * per_layer + tail
     # the step wrote row n_past of both caches and nothing else
     kc_ref, vc_ref = kc.copy(), vc.copy()
     _ref_step(w, hp, kc_ref, vc_ref, 123, n_past)
@@ -115,7 +116,7 @@ def test_decode_from_an_empty_cache_over_several_tokens(gdev):
     vc = np.zeros_like(kc)
     for n_past, tok in enumerate([1, 400, 17, 17, 511]):
         ref = _ref_step(w, hp, kc, vc, tok, n_past)
-        dec.decode(tok, n_past, False)
+        dec.decode(tok, n_past, 2 * (n_past % 2))   # alternate one-kernel-per-op and grouped steps on one cache
         _check(dec.logits(), ref, 1e-4)
     dec.close()
 
@@ -127,16 +128,16 @@ def test_graph_replays_equal_the_eager_step(gdev):
     kc = rng.standard_normal((hp["n_layer"], hp["n_ctx"], hp["n_embd"])).astype(np.float32)
     dec = g.LlamaDecoder(gdev, **hp)
     _load(dec, w, kc, kc[::-1].copy())
-    dec.decode(9, 20, True)
+    dec.decode(9, 20, 2)
     eager = dec.logits()
-    dec.capture(9, 20, True)
+    dec.capture(9, 20, 2)
     for i in range(4):
         dec.replay()
         assert np.array_equal(dec.logits(), eager), i
         # eager work and synchronisation between the replays
         dec.decode(9 + i, 30 + i, False)        # appends rows the recorded step (21 keys) never reads
         assert not np.array_equal(dec.logits(), eager)
-        dec.decode(9, 20, True)                 # puts token 9 / position 20 back into the device-side inputs
+        dec.decode(9, 20, 2)                    # puts token 9 / position 20 back into the device-side inputs
     dec.close()
 
 
