@@ -1,0 +1,244 @@
+// Attention of one decode step over an f32 KV cache, as one streaming pass.
+//
+// In galois's op vocabulary a decode step's attention is rope_custom(q), rope_custom(k), cpy(k -> cache row),
+// cpy(v -> cache row), matmul(K^T, q), scale, soft_max, matmul(V, p) (launchers src/cuda.rs:1257-1356, 1382-1595,
+// 698-782, 1597-1663).  Issued one by one these are nine launches that read the 64 MB of one layer's cache at
+// a third of the HBM rate, most of the time being launch gaps.  Here the same arithmetic runs in two launches:
+//
+//   attn_decode_partial: a workgroup owns 128 consecutive keys of one head.  It rotates its head's q (every
+//     workgroup of the head does, it is 128 floats), and the workgroup that owns position n_past also rotates
+//     the new k and writes k and v into row n_past of the caches.  Scores = scale * (k . q) go to LDS; the
+//     workgroup takes their maximum m, p = exp(score - m), the sum of p and the partial output sum p * v, and
+//     writes (m, sum, partial output) to the context's scratch block;
+//   attn_decode_combine: per head, rescales the partials to the global maximum, adds them in split order and
+//     divides by the total: out = softmax(scores) . V exactly as the three separate ops define it, up to the
+//     order of the f32 additions.
+//
+// A lane owns 4 consecutive floats of a head; head_dim / 4 lanes cover one key, so a wave-load of 16 bytes per
+// lane reads 64 / (head_dim / 4) whole cache rows of the head (512 contiguous bytes each for head_dim 128).
+#include "common.h"
+
+namespace {
+
+constexpr int AT_THREADS = 256;
+constexpr int AT_KEYS = 128;  // keys per workgroup
+
+template <int CTRL>
+__device__ __forceinline__ float at_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over aligned groups of LANES lanes (16 or 32); every lane of a group ends with its total.
+template <int LANES>
+__device__ __forceinline__ float at_group_sum(float v) {
+    v += at_dpp<0xB1>(v);   // quad_perm(1,0,3,2)
+    v += at_dpp<0x4E>(v);   // quad_perm(2,3,0,1)
+    v += at_dpp<0x141>(v);  // row_half_mirror
+    v += at_dpp<0x140>(v);  // row_mirror
+    if (LANES >= 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
+__device__ __forceinline__ float at_wave_max(float v) {
+    v = fmaxf(v, at_dpp<0xB1>(v));
+    v = fmaxf(v, at_dpp<0x4E>(v));
+    v = fmaxf(v, at_dpp<0x141>(v));
+    v = fmaxf(v, at_dpp<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+__device__ __forceinline__ float at_wave_sum(float v) {
+    v += at_dpp<0xB1>(v);
+    v += at_dpp<0x4E>(v);
+    v += at_dpp<0x141>(v);
+    v += at_dpp<0x140>(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// Rotation of the lane's two adjacent pairs (rope.cu:3-28, mode 0): pair i of the head by
+// theta = pos * freq_scale * theta_scale^i.
+struct at_rot {
+    float c0, s0, c1, s1;
+    __device__ __forceinline__ float4 apply(float4 x) const {
+        return make_float4(x.x * c0 - x.y * s0, x.x * s0 + x.y * c0, x.z * c1 - x.w * s1, x.z * s1 + x.w * c1);
+    }
+};
+
+// Record of one (head, split) in the scratch block: m, sum, 2 unused floats, then head_dim partial outputs.
+template <int LPR>
+__global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *__restrict__ q, const float *__restrict__ k,
+                                                                  const float *__restrict__ v, float *__restrict__ kc,
+                                                                  float *__restrict__ vc, float *__restrict__ part,
+                                                                  float *__restrict__ out, int H, int L,
+                                                                  const int32_t *__restrict__ pos, float freq_scale,
+                                                                  float theta_scale, float scale) {
+    constexpr int D = LPR * 4, RPL = 64 / LPR, WAVES = AT_THREADS / 64;
+    constexpr int KPW = AT_KEYS / WAVES;  // keys per wave
+    constexpr int U = KPW / RPL;          // wave-loads per wave, all in flight
+    __shared__ float sc[AT_KEYS];
+    __shared__ float4 ored[WAVES][LPR];
+    __shared__ float sred[WAVES];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / LPR, kl = lane % LPR;
+    const int h = blockIdx.y, s = blockIdx.x, S = gridDim.x;
+    const int l0 = s * AT_KEYS, l1 = min(L, l0 + AT_KEYS), nl = l1 - l0;
+    const size_t E = (size_t)H * D;
+    const size_t hoff = (size_t)h * D + kl * 4;
+
+    // this position's rotation for the lane's pairs 2 kl and 2 kl + 1
+    at_rot rot;
+    {
+        const float p0 = (float)pos[0] * freq_scale;
+        sincosf(p0 * powf(theta_scale, (float)(2 * kl)), &rot.s0, &rot.c0);
+        sincosf(p0 * powf(theta_scale, (float)(2 * kl + 1)), &rot.s1, &rot.c1);
+    }
+    const float4 qv = rot.apply(*reinterpret_cast<const float4 *>(q + hoff));
+    const int lnew = L - 1;  // the position being appended
+
+    // ---- scores of the workgroup's keys
+    {
+        float4 kv[U];
+        const int kbase = l0 + wave * KPW + sub;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int l = kbase + u * RPL;
+            const int lc = min(l, l1 - 1);
+            if (lc == lnew) {  // not in the cache yet: rotate it, use it, write it
+                kv[u] = rot.apply(*reinterpret_cast<const float4 *>(k + hoff));
+                if (l == lnew) *reinterpret_cast<float4 *>(kc + (size_t)lnew * E + hoff) = kv[u];
+            } else {
+                kv[u] = *reinterpret_cast<const float4 *>(kc + (size_t)lc * E + hoff);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float acc = kv[u].x * qv.x;
+            acc = __builtin_fmaf(kv[u].y, qv.y, acc);
+            acc = __builtin_fmaf(kv[u].z, qv.z, acc);
+            acc = __builtin_fmaf(kv[u].w, qv.w, acc);
+            acc = at_group_sum<LPR>(acc);
+            if (kl == 0) sc[wave * KPW + u * RPL + sub] = acc * scale;
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax numerators relative to the workgroup's own maximum
+    float m;
+    {
+        const float ninf = -__builtin_inff();
+        const float a = lane < nl ? sc[lane] : ninf, b = lane + 64 < nl ? sc[lane + 64] : ninf;
+        m = at_wave_max(fmaxf(a, b));
+    }
+    __syncthreads();  // every wave has read the scores
+    if (threadIdx.x < AT_KEYS) sc[threadIdx.x] = (int)threadIdx.x < nl ? expf(sc[threadIdx.x] - m) : 0.0f;
+    __syncthreads();
+
+    // ---- partial output: sum of p * v over the workgroup's keys
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    {
+        float4 vv[U];
+        const int kbase = l0 + wave * KPW + sub;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int l = kbase + u * RPL;
+            const int lc = min(l, l1 - 1);
+            if (lc == lnew) {
+                vv[u] = *reinterpret_cast<const float4 *>(v + hoff);
+                if (l == lnew) *reinterpret_cast<float4 *>(vc + (size_t)lnew * E + hoff) = vv[u];
+            } else {
+                vv[u] = *reinterpret_cast<const float4 *>(vc + (size_t)lc * E + hoff);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float p = sc[wave * KPW + u * RPL + sub];  // 0 for keys past the end
+            acc.x = __builtin_fmaf(vv[u].x, p, acc.x);
+            acc.y = __builtin_fmaf(vv[u].y, p, acc.y);
+            acc.z = __builtin_fmaf(vv[u].z, p, acc.z);
+            acc.w = __builtin_fmaf(vv[u].w, p, acc.w);
+        }
+    }
+    // the RPL keys of a wave-load sit LPR lanes apart
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off, 64);
+        acc.y += __shfl_xor(acc.y, off, 64);
+        acc.z += __shfl_xor(acc.z, off, 64);
+        acc.w += __shfl_xor(acc.w, off, 64);
+    }
+    if (lane < LPR) ored[wave][lane] = acc;
+    const float psum = at_wave_sum((lane < nl ? sc[lane] : 0.0f) + (lane + 64 < nl ? sc[lane + 64] : 0.0f));
+    if (lane == 0) sred[wave] = psum;  // every wave holds the same total; wave 0's is used
+    __syncthreads();
+    if (wave == 0 && lane < LPR) {
+        float4 o = ored[0][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) {
+            const float4 t = ored[w][lane];
+            o.x += t.x, o.y += t.y, o.z += t.z, o.w += t.w;
+        }
+        const float tot = sred[0];
+        if (S == 1) {  // a single split is the whole softmax
+            const float inv = 1.0f / tot;
+            *reinterpret_cast<float4 *>(out + (size_t)h * D + lane * 4) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+        } else {
+            float *rec = part + ((size_t)h * S + s) * (D + 4);
+            if (lane == 0) rec[0] = m, rec[1] = tot;
+            *reinterpret_cast<float4 *>(rec + 4 + lane * 4) = o;
+        }
+    }
+}
+
+// One workgroup per head, one thread per output element.
+__global__ void attn_decode_combine(const float *__restrict__ part, float *__restrict__ out, int D, int S) {
+    const int h = blockIdx.x, d = threadIdx.x;
+    const float *rec = part + (size_t)h * S * (D + 4);
+    float M = -__builtin_inff();
+    for (int s = 0; s < S; s++) M = fmaxf(M, rec[(size_t)s * (D + 4)]);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < S; s++) {
+        const float *r = rec + (size_t)s * (D + 4);
+        const float w = expf(r[0] - M);
+        den = __builtin_fmaf(w, r[1], den);
+        num = __builtin_fmaf(w, r[4 + d], num);
+    }
+    out[(size_t)h * D + d] = num / den;
+}
+
+}  // namespace
+
+extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
+                                              float *k_cache, float *v_cache, float *out, int32_t n_head,
+                                              int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
+                                              float theta_scale, float scale) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, q && k && v && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, "attn_decode_f32");
+    GH_REQUIRE(ctx, n_head > 0 && n_head <= 65535 && n_past >= 0 && n_past < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
+               "attn_decode_f32: n_head in 1..65535, n_past >= 0");
+    GH_REQUIRE(ctx, head_dim == 64 || head_dim == 128, GALOIS_HIP_E_UNSUPPORTED, "attn_decode_f32: head_dim 64 or 128");
+    GH_REQUIRE(ctx, gh_aligned(q, 16) && gh_aligned(k, 16) && gh_aligned(v, 16) && gh_aligned(k_cache, 16) &&
+                        gh_aligned(v_cache, 16) && gh_aligned(out, 16) && gh_aligned(pos, 4),
+               GALOIS_HIP_E_ALIGN, "attn_decode_f32: 16-byte aligned vectors and caches");
+    const int L = n_past + 1;
+    const int S = (L + AT_KEYS - 1) / AT_KEYS;
+    GH_REQUIRE(ctx, S == 1 || ((int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr),
+               GALOIS_HIP_E_UNSUPPORTED, "attn_decode_f32: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
+                                         "results must fit the context's 4 MB scratch block");
+    GH_BIND(ctx);
+    float *part = (float *)ctx->scratch;
+    const dim3 grid((unsigned)S, (unsigned)n_head), block(AT_THREADS);
+    if (head_dim == 128)
+        hipLaunchKernelGGL(attn_decode_partial<32>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, out,
+                           n_head, L, pos, freq_scale, theta_scale, scale);
+    else
+        hipLaunchKernelGGL(attn_decode_partial<16>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, out,
+                           n_head, L, pos, freq_scale, theta_scale, scale);
+    if (S > 1)
+        hipLaunchKernelGGL(attn_decode_combine, dim3((unsigned)n_head), dim3((unsigned)head_dim), 0, ctx->stream, part, out,
+                           head_dim, S);
+    GH_LAUNCH_CHECK(ctx, "attn_decode_f32 launch");
+}

@@ -69,6 +69,28 @@ GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
     return dev->check(galois_hip_dequantize_mul_mat_vec_q4_0_group(dev->ctx(), it, (int32_t)items.size()));
 }
 
+GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
+                           Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale) {
+    std::shared_ptr<CudaDevice> dev;
+    for (const Tensor *t : {&q, &k, &v, (const Tensor *)&k_cache, (const Tensor *)&v_cache, &pos, (const Tensor *)&out}) {
+        if (!t->device().is_gpu()) return err(GError::Unimplemented, "galois_attn_decode: Gpu tensors only");
+        if (!dev) dev = t->device().gpu;
+        if (t->device().gpu != dev) return err(GError::Unimplemented, "galois_attn_decode: one device");
+        if (!t->dim().ggml_is_contiguous(t->dtype())) return err(GError::Unimplemented, "galois_attn_decode: contiguous tensors only");
+        if (t->dtype() != (t == &pos ? GGmlType::I32 : GGmlType::F32)) return err(GError::Unimplemented, "galois_attn_decode: F32 tensors, I32 pos");
+    }
+    if (op.mode != 0) return err(GError::Unimplemented, "galois_attn_decode: rope mode 0 only (src/cuda.rs:1336-1340)");
+    const size_t E = q.dim().elem_count();
+    if (n_head == 0 || E % n_head != 0 || op.n_dims != E / n_head || k.dim().elem_count() != E || v.dim().elem_count() != E ||
+        out.dim().elem_count() != E || k_cache.dim().shape[0] != E || v_cache.dim().shape[0] != E || pos.dim().elem_count() != 1 ||
+        n_past < 0 || (size_t)n_past >= k_cache.dim().shape[1] || (size_t)n_past >= v_cache.dim().shape[1])
+        return err(GError::ShapeError, "galois_attn_decode: q, k, v, out of n_head * n_dims elements, caches [that, n_ctx], n_past < n_ctx");
+    const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);  // as galois_rope_custom derives it (src/cuda.rs:1327)
+    return dev->check(galois_hip_attn_decode_f32(dev->ctx(), (const float *)q.data(), (const float *)k.data(), (const float *)v.data(),
+                                                 (float *)k_cache.data(), (float *)v_cache.data(), (float *)out.data(), (int32_t)n_head,
+                                                 (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
+}
+
 static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t ne1 = 0, size_t ne2 = 0) {
     const size_t shape[3] = {ne0, ne1, ne2};
     return Tensor::zeros(ne2 ? 3 : (ne1 ? 2 : 1), shape, ty, dev, t);
@@ -189,6 +211,20 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
             G_TRY(galois_matmul(l.wq, a_, q_));
             G_TRY(galois_matmul(l.wk, a_, k_));
             G_TRY(galois_matmul(l.wv, a_, v_)); ops += 3;
+        }
+        if (fused >= 3) {  // the eight attention ops as two launches, then the grouped tail of the layer
+            G_TRY(galois_attn_decode(rope, q_, k_, v_, l.k_cache, l.v_cache, pos_, ao_, H, n_past, *(const float *)scale_.data()));
+            ops += L > 128 ? 2 : 1;
+            MatvecItem mo = item(l.wo, ao_, x1_);
+            mo.residual = &x_;
+            G_TRY(galois_matvec_group({mo})); ops++;
+            MatvecItem mg = item(l.w_gate, x1_, h_);
+            mg.w_up = &l.w_up, mg.norm_weight = &l.ffn_norm;
+            G_TRY(galois_matvec_group({mg})); ops++;
+            MatvecItem md = item(l.w_down, h_, x_);
+            md.residual = &x1_;
+            G_TRY(galois_matvec_group({md})); ops++;
+            continue;
         }
         Tensor qv, kv;
         const size_t hs[3] = {D, H, 1};

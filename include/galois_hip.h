@@ -211,6 +211,19 @@ int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const i
 int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K, int32_t N,
                                int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2);
 
+/* Attention of one decode step over an f32 KV cache in two launches instead of the nine of the op sequence
+ * rope_custom(q), rope_custom(k), cpy(k -> cache), cpy(v -> cache), matmul(K^T, q), scale, soft_max, matmul(V, p)
+ * (src/cuda.rs:1257-1356, 1382-1595, 698-782, 1597-1663), with the same arithmetic up to the order of f32 sums:
+ *   q, k, v: this token's n_head * head_dim projections (not yet rotated); pos: its position (one int32 on the device,
+ *   as rope_f32 takes it); rotation parameters as rope_f32 (mode 0, n_dims = head_dim);
+ *   k_cache, v_cache: [n_ctx][n_head * head_dim] f32; row n_past receives rope(k) and v;
+ *   out[h * head_dim + d] = sum_l softmax_l(scale * rope(q)_h . K[l]_h) * V[l][h * head_dim + d] over l = 0 .. n_past.
+ * head_dim 64 or 128; all pointers 16-byte aligned; partial results live in the context's scratch block, which bounds
+ * n_head * ceil((n_past + 1) / 128) * (head_dim + 4) by 2^20. */
+int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, float *k_cache,
+                                   float *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
+                                   const int32_t *pos, float freq_scale, float theta_scale, float scale);
+
 #ifdef __cplusplus
 }
 #endif

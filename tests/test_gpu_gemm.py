@@ -34,10 +34,11 @@ def _case(seed, m, k, n):
     return oracle.quantize_q4_0(w), x
 
 
-def test_gemm_layout_probe(dev):
+@pytest.mark.parametrize("k,n,m", [(64, 160, 130), (256, 200, 130), (1024, 353, 257)])
+def test_gemm_layout_probe(dev, k, n, m):
     """One-hot activations pick single dequantised weights: catches any transposed or permuted
-    operand / accumulator layout exactly (values are exactly representable in fp16)."""
-    k, n, m = 64, 160, 130
+    operand / accumulator layout exactly (values are exactly representable in fp16).  K = 64 runs the
+    generic kernel, the multiples of 256 the main one (several k-stages, ragged M and N tiles)."""
     rng = np.random.default_rng(0)
     nib = rng.integers(0, 16, (n, k // 32, 32))
     qs = (nib[..., :16] | (nib[..., 16:] << 4)).astype(np.uint8)
@@ -52,7 +53,8 @@ def test_gemm_layout_probe(dev):
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 32, 1), (2, 64, 3), (63, 96, 65), (64, 128, 64), (65, 256, 129),
-                                   (128, 512, 128), (129, 4096, 257), (512, 1024, 384)])
+                                   (128, 512, 128), (129, 4096, 257), (512, 1024, 384), (1, 256, 1), (300, 768, 177),
+                                   (16, 2048, 176), (17, 11008, 100)])
 def test_gemm_shapes_vs_oracle(dev, m, k, n):
     wq, x = _case(m * 7 + k + n, m, k, n)
     ref = oracle.mul_mat_q4_0_f32(wq, x)

@@ -87,11 +87,12 @@ def test_decode_step_matches_oracle_with_a_filled_cache(gdev):
     dec = g.LlamaDecoder(gdev, **hp)
     _load(dec, w, kc, vc)
     ref = _ref_step(w, hp, kc.copy(), vc.copy(), 123, n_past)
-    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1)):
+    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1), (3, 5, 1)):
         _load(dec, w, kc, vc)
         dec.decode(123, n_past, fused)
         _check(dec.logits(), ref, 1e-4)
-        # launches: embedding lookup + per layer + final norm and lm head (fused = 2: grouped products, 12 per layer)
+        # launches: embedding lookup + per layer + final norm and lm head (fused = 2: grouped products, 12 per layer;
+        # fused = 3: attention in one launch too while n_past + 1 <= 128 keys, two beyond)
         assert dec.ops_per_step() == 1 + hp["n_layer"] * per_layer + tail
     # the step wrote row n_past of both caches and nothing else
     kc_ref, vc_ref = kc.copy(), vc.copy()
@@ -116,7 +117,7 @@ def test_decode_from_an_empty_cache_over_several_tokens(gdev):
     vc = np.zeros_like(kc)
     for n_past, tok in enumerate([1, 400, 17, 17, 511]):
         ref = _ref_step(w, hp, kc, vc, tok, n_past)
-        dec.decode(tok, n_past, 2 * (n_past % 2))   # alternate one-kernel-per-op and grouped steps on one cache
+        dec.decode(tok, n_past, (0, 3, 2, 1, 3)[n_past])   # every launch plan in turn, on one cache
         _check(dec.logits(), ref, 1e-4)
     dec.close()
 
