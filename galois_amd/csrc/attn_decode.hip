@@ -89,6 +89,23 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
     const size_t E = (size_t)H * D;
     const size_t hoff = (size_t)h * D + kl * 4;
 
+    const int lnew = L - 1;  // the position being appended
+    const int kbase = l0 + wave * KPW + sub;
+
+    // ---- every request of the workgroup goes out first: its keys and values (the new position's come from k and
+    // v, it is not in the cache yet), then q; the rotation is computed while they are in flight
+    float4 kv[U], vv[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int lc = min(kbase + u * RPL, l1 - 1);
+        kv[u] = *reinterpret_cast<const float4 *>(lc == lnew ? k + hoff : kc + (size_t)lc * E + hoff);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int lc = min(kbase + u * RPL, l1 - 1);
+        vv[u] = *reinterpret_cast<const float4 *>(lc == lnew ? v + hoff : vc + (size_t)lc * E + hoff);
+    }
+    const float4 qraw = *reinterpret_cast<const float4 *>(q + hoff);
     // this position's rotation for the lane's pairs 2 kl and 2 kl + 1
     at_rot rot;
     {
@@ -96,33 +113,25 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
         sincosf(p0 * powf(theta_scale, (float)(2 * kl)), &rot.s0, &rot.c0);
         sincosf(p0 * powf(theta_scale, (float)(2 * kl + 1)), &rot.s1, &rot.c1);
     }
-    const float4 qv = rot.apply(*reinterpret_cast<const float4 *>(q + hoff));
-    const int lnew = L - 1;  // the position being appended
+    const float4 qv = rot.apply(qraw);
 
     // ---- scores of the workgroup's keys
-    {
-        float4 kv[U];
-        const int kbase = l0 + wave * KPW + sub;
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int l = kbase + u * RPL;
-            const int lc = min(l, l1 - 1);
-            if (lc == lnew) {  // not in the cache yet: rotate it, use it, write it
-                kv[u] = rot.apply(*reinterpret_cast<const float4 *>(k + hoff));
-                if (l == lnew) *reinterpret_cast<float4 *>(kc + (size_t)lnew * E + hoff) = kv[u];
-            } else {
-                kv[u] = *reinterpret_cast<const float4 *>(kc + (size_t)lc * E + hoff);
+    for (int u = 0; u < U; u++) {
+        const int l = kbase + u * RPL;
+        if (min(l, l1 - 1) == lnew) {  // rotate the new key; the lanes that own it write both cache rows
+            kv[u] = rot.apply(kv[u]);
+            if (l == lnew) {
+                *reinterpret_cast<float4 *>(kc + (size_t)lnew * E + hoff) = kv[u];
+                *reinterpret_cast<float4 *>(vc + (size_t)lnew * E + hoff) = vv[u];
             }
         }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            float acc = kv[u].x * qv.x;
-            acc = __builtin_fmaf(kv[u].y, qv.y, acc);
-            acc = __builtin_fmaf(kv[u].z, qv.z, acc);
-            acc = __builtin_fmaf(kv[u].w, qv.w, acc);
-            acc = at_group_sum<LPR>(acc);
-            if (kl == 0) sc[wave * KPW + u * RPL + sub] = acc * scale;
-        }
+        float acc = kv[u].x * qv.x;
+        acc = __builtin_fmaf(kv[u].y, qv.y, acc);
+        acc = __builtin_fmaf(kv[u].z, qv.z, acc);
+        acc = __builtin_fmaf(kv[u].w, qv.w, acc);
+        acc = at_group_sum<LPR>(acc);
+        if (kl == 0) sc[wave * KPW + u * RPL + sub] = acc * scale;
     }
     __syncthreads();
 
@@ -137,30 +146,15 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
     if (threadIdx.x < AT_KEYS) sc[threadIdx.x] = (int)threadIdx.x < nl ? expf(sc[threadIdx.x] - m) : 0.0f;
     __syncthreads();
 
-    // ---- partial output: sum of p * v over the workgroup's keys
+    // ---- partial output: sum of p * v over the workgroup's keys (p is 0 for keys past the end)
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    {
-        float4 vv[U];
-        const int kbase = l0 + wave * KPW + sub;
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int l = kbase + u * RPL;
-            const int lc = min(l, l1 - 1);
-            if (lc == lnew) {
-                vv[u] = *reinterpret_cast<const float4 *>(v + hoff);
-                if (l == lnew) *reinterpret_cast<float4 *>(vc + (size_t)lnew * E + hoff) = vv[u];
-            } else {
-                vv[u] = *reinterpret_cast<const float4 *>(vc + (size_t)lc * E + hoff);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const float p = sc[wave * KPW + u * RPL + sub];  // 0 for keys past the end
-            acc.x = __builtin_fmaf(vv[u].x, p, acc.x);
-            acc.y = __builtin_fmaf(vv[u].y, p, acc.y);
-            acc.z = __builtin_fmaf(vv[u].z, p, acc.z);
-            acc.w = __builtin_fmaf(vv[u].w, p, acc.w);
-        }
+    for (int u = 0; u < U; u++) {
+        const float p = sc[wave * KPW + u * RPL + sub];
+        acc.x = __builtin_fmaf(vv[u].x, p, acc.x);
+        acc.y = __builtin_fmaf(vv[u].y, p, acc.y);
+        acc.z = __builtin_fmaf(vv[u].z, p, acc.z);
+        acc.w = __builtin_fmaf(vv[u].w, p, acc.w);
     }
     // the RPL keys of a wave-load sit LPR lanes apart
 #pragma unroll
@@ -193,18 +187,43 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
     }
 }
 
-// One workgroup per head, one thread per output element.
+// One workgroup per head, one thread per output element.  The split maxima and sums are fetched by S threads at
+// once and the weights exp(m_s - M) shared through LDS; the partial outputs are then read eight splits at a time.
+constexpr int AT_MAX_SPLITS = 1024;
 __global__ void attn_decode_combine(const float *__restrict__ part, float *__restrict__ out, int D, int S) {
-    const int h = blockIdx.x, d = threadIdx.x;
+    __shared__ float w[AT_MAX_SPLITS];
+    __shared__ float red[2][2];
+    const int h = blockIdx.x, d = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
     const float *rec = part + (size_t)h * S * (D + 4);
-    float M = -__builtin_inff();
-    for (int s = 0; s < S; s++) M = fmaxf(M, rec[(size_t)s * (D + 4)]);
-    float num = 0.0f, den = 0.0f;
-    for (int s = 0; s < S; s++) {
-        const float *r = rec + (size_t)s * (D + 4);
-        const float w = expf(r[0] - M);
-        den = __builtin_fmaf(w, r[1], den);
-        num = __builtin_fmaf(w, r[4 + d], num);
+    float mx = -__builtin_inff();
+    for (int s = d; s < S; s += blockDim.x) {
+        const float2 ms = *reinterpret_cast<const float2 *>(rec + (size_t)s * (D + 4));
+        w[s] = ms.x;
+        mx = fmaxf(mx, ms.x);
+    }
+    mx = at_wave_max(mx);
+    if (lane == 0) red[0][wave] = mx;
+    __syncthreads();
+    const float M = nwaves == 1 ? red[0][0] : fmaxf(red[0][0], red[0][1]);
+    float den = 0.0f;
+    for (int s = d; s < S; s += blockDim.x) {
+        const float ws = expf(w[s] - M);
+        w[s] = ws;
+        den = __builtin_fmaf(ws, rec[(size_t)s * (D + 4) + 1], den);
+    }
+    den = at_wave_sum(den);
+    if (lane == 0) red[1][wave] = den;
+    __syncthreads();
+    den = nwaves == 1 ? red[1][0] : red[1][0] + red[1][1];
+    float num = 0.0f;
+    for (int s0 = 0; s0 < S; s0 += 8) {
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] = rec[(size_t)min(s0 + j, S - 1) * (D + 4) + 4 + d];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (s0 + j < S) num = __builtin_fmaf(w[s0 + j], o[j], num);
     }
     out[(size_t)h * D + d] = num / den;
 }
@@ -225,7 +244,7 @@ extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *
                GALOIS_HIP_E_ALIGN, "attn_decode_f32: 16-byte aligned vectors and caches");
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
-    GH_REQUIRE(ctx, S == 1 || ((int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr),
+    GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && (int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr),
                GALOIS_HIP_E_UNSUPPORTED, "attn_decode_f32: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
                                          "results must fit the context's 4 MB scratch block");
     GH_BIND(ctx);
