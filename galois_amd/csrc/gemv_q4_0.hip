@@ -17,6 +17,8 @@
 #include "common.h"
 #include "gemv_xprep.h"
 
+#include <type_traits>
+
 // Phase timestamps for tuning builds (-DGEMV_TIMING): one s_memtime per phase per wave.
 #ifdef GEMV_TIMING
 __device__ unsigned long long *g_gemv_tbuf;
@@ -454,8 +456,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     __syncthreads();
     GH_TSTAMP(4);
 
-    for (int g = 0; g < groups; g++, row0 += WAVES * rw) {
-        if (g > 0 && row0 >= N) break;  // wave-uniform
+    // One group of rows.  The first group's first slots are the ones requested before the preparation; it is
+    // peeled off the loop so that those registers are not kept alive through the later groups.
+    auto do_group = [&](auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
         for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
             const bool act = sl < ns;
             const int s_ld = min(sl, ns - 1);
@@ -475,7 +479,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                 sB = __builtin_bit_cast(float, sc.y);
             }
             q4_slot q[R];
-            if (g == 0 && sl == lane) {
+            if (FIRST && sl == lane) {
 #pragma unroll
                 for (int j = 0; j < R; j++) q[j] = q0[j];
             } else {
@@ -516,6 +520,12 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         }
 #pragma unroll
         for (int j = 0; j < R; j++) acc[j] = 0.0f;
+    };
+    do_group(std::true_type{});
+    for (int g = 1; g < groups; g++) {
+        row0 += WAVES * rw;
+        if (row0 >= N) break;  // wave-uniform
+        do_group(std::false_type{});
     }
     GH_TSTAMP(6);
 }
@@ -594,12 +604,12 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     if (cfg != 1 && cfg != 4) cfg = (!any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16) ? 1 : 4;
     if (any_dual) cfg = 4;
     const int slots_per_wg = 16;  // WAVES * R of both shapes
+    // One row group per wave: measured, working through two or four groups per wave (which would amortise the
+    // activation preparation) loses more to the coarser split of the launch than it saves at every LLaMA-7B shape.
     int64_t blocks = 0;
     for (int i = 0; i < n_items; i++) {
-        // more rows per workgroup when there are plenty: the preparation is paid once per workgroup
-        const int64_t wgs1 = ((int64_t)items[i].nrows * (items[i].vx_up ? 2 : 1) + slots_per_wg - 1) / slots_per_wg;
         int groups = ctx->gemv_units_per_wave;
-        if (groups <= 0) groups = wgs1 >= 4 * (int64_t)ctx->n_cu ? 2 : 1;  // measured: 9 % on the 32000-row matrix
+        if (groups <= 0) groups = 1;
         groups = groups < 1 ? 1 : (groups > 4 ? 4 : groups);
         a.item[i].groups = groups;
         const int64_t rows_per_wg = (items[i].vx_up ? slots_per_wg / 2 : slots_per_wg) * groups;
@@ -633,8 +643,7 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, c
         // activation preparation is spread over 1024 threads; more rows -> 8 waves x 2 rows, several
         // workgroups resident per CU so one's preparation overlaps another's streaming.
         int cfg = ctx->gemv_config;
-        // many rows: the group kernel's two row groups per wave halve the preparation per row
-        if ((cfg == 6 || (cfg == 0 && nrows >= 64 * ctx->n_cu)) && ncols <= 64 * GG_MAX_SLOTS) {
+        if (cfg == 6 && ncols <= 64 * GG_MAX_SLOTS) {
             galois_hip_gemv_item it;
             memset(&it, 0, sizeof(it));
             it.vx = vx, it.y = y, it.dst = dst, it.ncols = ncols, it.nrows = nrows;
