@@ -563,8 +563,8 @@ void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, in
         else
             hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, false>), grid, block, lds, ctx->stream, a);
     } else {
-        if (norm)
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, true>), grid, block, lds, ctx->stream, a);
+        if (norm)  // the normalising preparation of a long vector needs more than 64 registers
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, (OCC > 4 ? 4 : OCC), true>), grid, block, lds, ctx->stream, a);
         else
             hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, false>), grid, block, lds, ctx->stream, a);
     }
@@ -601,8 +601,8 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     bool any_dual = false;
     for (int i = 0; i < n_items; i++) any_dual |= items[i].vx_up != nullptr;
     int cfg = ctx->gemv_config;
-    if (cfg != 1 && cfg != 4) cfg = (!any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16) ? 1 : 4;
-    if (any_dual) cfg = 4;
+    if (cfg != 1 && cfg != 4 && cfg != 7) cfg = (!any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16) ? 1 : 4;
+    if (any_dual && cfg == 1) cfg = 4;
     const int slots_per_wg = 16;  // WAVES * R of both shapes
     // One row group per wave: measured, working through two or four groups per wave (which would amortise the
     // activation preparation) loses more to the coarser split of the launch than it saves at every LLaMA-7B shape.
@@ -620,6 +620,8 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     GH_BIND(ctx);
     if (cfg == 1)
         launch_group_cfg<5, 1, 16, 4>(ctx, a, (unsigned)blocks, max_slots, norm);
+    else if (cfg == 7)
+        launch_group_cfg<5, 2, 8, 8>(ctx, a, (unsigned)blocks, max_slots, norm);
     else
         launch_group_cfg<5, 2, 8, 4>(ctx, a, (unsigned)blocks, max_slots, norm);
     GH_LAUNCH_CHECK(ctx, what);
