@@ -236,35 +236,38 @@ __device__ __forceinline__ void gemm_store_raw(uint8_t *raw, int p, const gemm_r
 // (low nibbles) and the run k = 32b + 16 + 8jp .. (high nibbles).  The four lanes of a row write
 // 64 distinct bytes per store and neighbouring rows are 160 bytes apart, so the 16-byte stores of
 // eight consecutive lanes fall into 32 different banks.
-template <int J>
-__device__ __forceinline__ void gemm_dequant_stage(const uint8_t *raw, _Float16 *Bs, int p) {
-#ifdef GEMM_X_NO_DEQ
-    return;
-#endif
-    // all LDS reads of the thread's (up to) three tasks first, so that their latencies overlap
+// The raw bytes of a stage are read from LDS one stage ahead (gemm_stage_read) and turned into fp16
+// after the barrier (gemm_stage_write), so that the read latency is not on the path between two barriers.
+struct gemm_stage_regs {
     uint32_t dbits[3], w0[3], w1[3], w2[3];
+};
+
+template <int J>
+__device__ __forceinline__ void gemm_stage_read(gemm_stage_regs &r, const uint8_t *raw, int p) {
 #pragma unroll
     for (int it = 0; it < 3; it++) {
         const int q = p + 256 * it;
         if (it < 2 || q < GN * 4) {
             const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
             const int o = row * GRAW_STRIDE + 36 * J + 18 * b;  // the block: d at o, qs at o + 2
-            dbits[it] = *reinterpret_cast<const uint16_t *>(raw + o);
+            r.dbits[it] = *reinterpret_cast<const uint16_t *>(raw + o);
             const int qo = o + 2 + 8 * jp;                       // 4-byte aligned for b = 1, 2 mod 4 for b = 0
             const uint32_t *w = reinterpret_cast<const uint32_t *>(raw + (qo & ~3));
-            w0[it] = w[0], w1[it] = w[1], w2[it] = w[2];         // w2 of the very last task lies in the 16-byte pad
+            r.w0[it] = w[0], r.w1[it] = w[1], r.w2[it] = w[2];   // w2 of the very last task lies in the 16-byte pad
         }
     }
-    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs &r, _Float16 *Bs, int p) {
 #pragma unroll
     for (int it = 0; it < 3; it++) {
         const int q = p + 256 * it;
         if (it < 2 || q < GN * 4) {
             const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
             const uint32_t sh = b ? 0u : 16u;
-            const uint32_t q0 = __builtin_amdgcn_alignbit(w1[it], w0[it], sh);
-            const uint32_t q1 = __builtin_amdgcn_alignbit(w2[it], w1[it], sh);
-            const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t)dbits[it]);
+            const uint32_t q0 = __builtin_amdgcn_alignbit(r.w1[it], r.w0[it], sh);
+            const uint32_t q1 = __builtin_amdgcn_alignbit(r.w2[it], r.w1[it], sh);
+            const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t)r.dbits[it]);
             const half2_t d2 = {d, d};
             uint32_t lo[4], hi[4];
             deq_dword(q0, d2, lo, hi);
@@ -292,21 +295,28 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
     gemm_store_raw(raw0, p, rr);
     gemm_load_raw(W, wrow_bytes, N, n0, p, min(1, nsuper - 1), rr);
     __syncthreads();  // R
+    gemm_stage_regs s0, s1;
+    gemm_stage_read<0>(s0, raw0, p);
     for (int sup = 0; sup < nsuper; sup++) {
         const uint8_t *raw = (sup & 1) ? raw1 : raw0;
+        uint8_t *other = (sup & 1) ? raw0 : raw1;
         const int t = 4 * sup;
-        gemm_dequant_stage<0>(raw, smem + (t % GNBUF) * GB_HALFS, p);
+        gemm_stage_read<1>(s1, raw, p);
+        gemm_stage_write(s0, smem + (t % GNBUF) * GB_HALFS, p);
         __syncthreads();
-        gemm_dequant_stage<1>(raw, smem + ((t + 1) % GNBUF) * GB_HALFS, p);
+        gemm_stage_read<2>(s0, raw, p);
+        gemm_stage_write(s1, smem + ((t + 1) % GNBUF) * GB_HALFS, p);
         __syncthreads();
-        gemm_dequant_stage<2>(raw, smem + ((t + 2) % GNBUF) * GB_HALFS, p);
-        __syncthreads();
-        gemm_dequant_stage<3>(raw, smem + ((t + 3) % GNBUF) * GB_HALFS, p);
+        gemm_stage_read<3>(s1, raw, p);
+        gemm_stage_write(s0, smem + ((t + 2) % GNBUF) * GB_HALFS, p);
         // park the next piece (requested four stages ago) in the other raw buffer, whose last readers
         // passed a barrier three stages ago, and request the one after it
         GEMM_VMWAIT(0);
-        gemm_store_raw((sup & 1) ? raw0 : raw1, p, rr);
+        gemm_store_raw(other, p, rr);
         gemm_load_raw(W, wrow_bytes, N, n0, p, min(sup + 2, nsuper - 1), rr);
+        __syncthreads();
+        gemm_stage_read<0>(s0, other, p);  // the next piece's first stage (read again, unused, after the last piece)
+        gemm_stage_write(s1, smem + ((t + 3) % GNBUF) * GB_HALFS, p);
         __syncthreads();
     }
     // The last request is never consumed.  To the compiler an inline-asm load defines its destination at
