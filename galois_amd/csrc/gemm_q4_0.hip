@@ -141,7 +141,12 @@ __global__ __launch_bounds__(256) void gemm_q4_0_mfma_v1(const uint8_t *__restri
 //     against 384 MFMA cycles per SIMD.
 //   - blockIdx is mapped so that an XCD (blockIdx % 8) owns one 128-row panel of X and a
 //     contiguous range of weight tiles: X stays in that XCD's L2, W streams once per panel.
-constexpr int GM = 128, GN = 176, GK = 64;
+#ifndef GEMM_TILE_N
+#define GEMM_TILE_N 96
+#endif
+constexpr int GN = GEMM_TILE_N;           // 96: four consumer waves stacked in M (tile 256 x 96); 176: 2 x 2 (tile 128 x 176)
+constexpr int GM = GN == 96 ? 256 : 128;
+constexpr int GTASKS = (GN * 4 + 255) / 256;  // dequantisation tasks per producer thread and stage
 constexpr int GBSTRIDE = 80;                  // halfs per B row in LDS: 160-byte rows
 constexpr int GB_HALFS = GN * GBSTRIDE;       // 14,080 halfs (28,160 B) per stage buffer
 constexpr int GNBUF = 3;
@@ -239,15 +244,15 @@ __device__ __forceinline__ void gemm_store_raw(uint8_t *raw, int p, const gemm_r
 // The raw bytes of a stage are read from LDS one stage ahead (gemm_stage_read) and turned into fp16
 // after the barrier (gemm_stage_write), so that the read latency is not on the path between two barriers.
 struct gemm_stage_regs {
-    uint32_t dbits[3], w0[3], w1[3], w2[3];
+    uint32_t dbits[GTASKS], w0[GTASKS], w1[GTASKS], w2[GTASKS];
 };
 
 template <int J>
 __device__ __forceinline__ void gemm_stage_read(gemm_stage_regs &r, const uint8_t *raw, int p) {
 #pragma unroll
-    for (int it = 0; it < 3; it++) {
+    for (int it = 0; it < GTASKS; it++) {
         const int q = p + 256 * it;
-        if (it < 2 || q < GN * 4) {
+        if ((it + 1) * 256 <= GN * 4 || q < GN * 4) {
             const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
             const int o = row * GRAW_STRIDE + 36 * J + 18 * b;  // the block: d at o, qs at o + 2
             r.dbits[it] = *reinterpret_cast<const uint16_t *>(raw + o);
@@ -260,9 +265,9 @@ __device__ __forceinline__ void gemm_stage_read(gemm_stage_regs &r, const uint8_
 
 __device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs &r, _Float16 *Bs, int p) {
 #pragma unroll
-    for (int it = 0; it < 3; it++) {
+    for (int it = 0; it < GTASKS; it++) {
         const int q = p + 256 * it;
-        if (it < 2 || q < GN * 4) {
+        if ((it + 1) * 256 <= GN * 4 || q < GN * 4) {
             const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
             const uint32_t sh = b ? 0u : 16u;
             const uint32_t q0 = __builtin_amdgcn_alignbit(r.w1[it], r.w0[it], sh);
@@ -466,10 +471,11 @@ __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict_
     const int mt = tile / n_tiles, nt = tile - mt * n_tiles;
     const int m0 = mt * GM, n0 = nt * GN;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // consumer waves 2 (M) x 2 (N): the left column owns 6 column tiles (96 wide), the right one 5 (80)
     if (wave >= 4)
         gemm_producer(smem, W, K, N, n0);
-    else if ((wave & 1) == 0)
+    else if (GN == 96)  // four consumer waves stacked in M, each 64 rows x 96 columns
+        gemm_consumer<6>(smem, Xh, Y, K, N, M, m0, n0, wave, 0);
+    else if ((wave & 1) == 0)  // 2 (M) x 2 (N): the left column owns 6 column tiles (96 wide), the right one 5 (80)
         gemm_consumer<6>(smem, Xh, Y, K, N, M, m0, n0, wave >> 1, 0);
     else
         gemm_consumer<5>(smem, Xh, Y, K, N, M, m0, n0, wave >> 1, 96);
