@@ -120,26 +120,27 @@ __global__ __launch_bounds__(256) void gemm_q4_0_mfma_v1(const uint8_t *__restri
         }
 }
 
-
 // ---------------------------------------------------------------------------------------
 // Main kernel: K % 256 == 0, W and X 16-byte aligned.
 //
 //   - X is rounded to fp16 once by f32_to_f16_tiles into a context-owned workspace, stored in the
 //     order the A operand of v_mfma_f32_16x16x32_f16 is held (per lane 8 consecutive k of one row),
 //     so a fragment is one contiguous KB: the consumer waves fetch their A fragments straight from
-//     global memory (the 4 MB panel stays in L2) one stage ahead, and X never touches LDS.
-//   - Workgroup tile 128 (M) x 176 (N), k-stage 64 (two Q4_0 blocks = one 36-byte slot per weight
-//     row).  11008 = 62.5 x 176, so the 512 x 11008 prefill is 4 x 63 = 252 workgroups: one round
-//     on 256 CUs.
-//   - 8 waves: 4 consumers as 2 (M) x 2 (N), wave tile 64 x 96 or 64 x 80 -> 4 x 6 (or 5) MFMA
-//     tiles with f32 accumulators in registers, and 4 producers that fetch the weights as whole
-//     144-byte row pieces (4 stages at a time), park them raw in LDS, and each stage dequantise
-//     one slot per row into an fp16 B tile.  Each SIMD hosts one wave of each kind.
+//     global memory (the 4 MB panel stays in L2) two stages ahead, and X never touches LDS.
+//   - Workgroup tile 256 (M) x 96 (N), k-stage 64 (two Q4_0 blocks = one 36-byte slot per weight
+//     row).  The 512 x 11008 prefill is 2 x 115 = 230 workgroups: one round on 256 CUs.
+//   - 8 waves: 4 consumers stacked in M, wave tile 64 x 96 -> 4 x 6 MFMA tiles with f32 accumulators
+//     in registers, and 4 producers that fetch the weights as whole 144-byte row pieces (4 stages at
+//     a time), park them raw in LDS, and each stage dequantise one slot per row into an fp16 B tile
+//     that all four consumers read.  Each SIMD hosts one wave of each kind.
+//     (-DGEMM_TILE_N=176 builds the earlier 128 x 176 tile with the consumers as 2 x 2.)
 //   - The fp16 B tile is triple-buffered, one barrier per stage: while the consumers multiply the
 //     second k-half of stage s they already hold the first half of stage s+1, and the producers
-//     write stage s+2.  LDS carries only B: 22 KB of fragment reads and 11 KB of writes per 32 k
-//     against 384 MFMA cycles per SIMD.
-//   - blockIdx is mapped so that an XCD (blockIdx % 8) owns one 128-row panel of X and a
+//     write stage s+2.  LDS carries only B.
+//   - A consumer wave has a single instruction stream, so whatever blocks it idles its SIMD's matrix
+//     pipe: its A requests and B fragment reads are issued one or two at a time between groups of
+//     six matrix instructions instead of in bursts.
+//   - blockIdx is mapped so that an XCD (blockIdx % 8) owns one 256-row panel of X and a
 //     contiguous range of weight tiles: X stays in that XCD's L2, W streams once per panel.
 #ifndef GEMM_TILE_N
 #define GEMM_TILE_N 96
@@ -294,6 +295,11 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
     uint8_t *raw0 = reinterpret_cast<uint8_t *>(smem + GNBUF * GB_HALFS);
     uint8_t *raw1 = raw0 + GRAW_BYTES;
 
+#ifdef GEMM_X_NO_PROD
+    __syncthreads();
+    for (int t = 0; t < nslots; t++) __syncthreads();
+    return;
+#endif
     gemm_raw_regs rr;
     gemm_load_raw(W, wrow_bytes, N, n0, p, 0, rr);
     GEMM_VMWAIT(0);
@@ -334,39 +340,41 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
 
 // ---- consumer side -----------------------------------------------------------------------
 // The A fragments are requested through inline assembly and waited for by hand.  Loads retire in
-// order, so "at most 8 younger loads outstanding" is the exact condition for the previous stage's
-// eight to have landed; left to the compiler, a load whose use is a loop iteration away is waited
-// for with vmcnt(0), which would also drain the prefetch just issued.
+// order, so "at most n younger loads outstanding" is the exact condition for an older one to have
+// landed; left to the compiler, a load whose use is a loop iteration away is waited for with
+// vmcnt(0), which would also drain the prefetches just issued.
 struct gemm_a_regs {
     u32x4_t c[8];  // [ks * 4 + i]: rows i*16 + lane%16 of the wave's 64, k = ks*32 + (lane/16)*8 ..
 };
 
-// Address = scalar base (the panel advanced to the stage: 2 KB per stage) + per-lane 32-bit offset
-// of the lane's piece in the first k-block of its 16-row group + immediate (second k-block: + 1 KB).
-__device__ __forceinline__ void gemm_load_a(gemm_a_regs &r, const _Float16 *xs, const uint32_t (&ro)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r.c[i]) : "v"(ro[i]), "s"(xs) : "memory");
-        asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(r.c[4 + i]) : "v"(ro[i]), "s"(xs) : "memory");
-    }
+// One fragment.  Address = scalar base xs (the panel advanced to the stage: 2 KB per stage) + per-lane
+// 32-bit offset ro of the lane's piece in the first k-block of its 16-row group + immediate (second
+// k-block, kh = 1: + 1 KB).
+__device__ __forceinline__ void gemm_load_a1(u32x4_t &dst, const _Float16 *xs, uint32_t ro, int kh) {
+    if (kh == 0)
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(ro), "s"(xs) : "memory");
+    else
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(dst) : "v"(ro), "s"(xs) : "memory");
 }
 
-// Waits until at most N loads are outstanding; naming the registers makes every later use of
-// them depend on the wait.
-#ifdef GEMM_X_HALF_A
-#define GEMM_WAIT_A(N, r) GEMM_WAIT_A_(4, r)
-#else
-#define GEMM_WAIT_A(N, r) GEMM_WAIT_A_(N, r)
-#endif
-#define GEMM_WAIT_A_(N, r)                                                                                   \
-    asm volatile("s_waitcnt vmcnt(" #N ")"                                                                   \
+// Drains the load counter; naming the registers keeps all of them allocated until here.
+#define GEMM_DRAIN_A(r)                                                                                      \
+    asm volatile("s_waitcnt vmcnt(0)"                                                                        \
                  : "+v"((r).c[0]), "+v"((r).c[1]), "+v"((r).c[2]), "+v"((r).c[3]), "+v"((r).c[4]), "+v"((r).c[5]), \
                    "+v"((r).c[6]), "+v"((r).c[7])::"memory")
 
+// Tuning builds: -DGEMM_X_NO_A / _NO_B / _NO_MFMA / _NO_PROD / _NO_STORE compile the kernel without its A
+// requests, B fragment reads, matrix instructions, producer work or result store (results are then
+// meaningless) to time what each part costs.
 #ifdef GEMM_X_NO_A
 #define GEMM_XA(...)
 #else
 #define GEMM_XA(...) __VA_ARGS__
+#endif
+#ifdef GEMM_X_NO_B
+#define GEMM_LDB(dst, ptr) asm volatile("" : "+v"(dst))
+#else
+#define GEMM_LDB(dst, ptr) dst = *reinterpret_cast<const half8_t *>(ptr)
 #endif
 #ifdef GEMM_X_NO_MFMA
 #define GEMM_MFMA(a, b, c) (c)
@@ -397,53 +405,75 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
     const int b_off = (ncol0 + (lane & 15)) * GBSTRIDE + (lane >> 4) * 8;
 
     gemm_a_regs a0, a1;
-    GEMM_XA(gemm_load_a(a0, Xh, ro);)
+    // requested in the order they are used: the waits below count younger requests
+    GEMM_XA(_Pragma("unroll") for (int g = 0; g < 8; g++) gemm_load_a1(a0.c[g], Xh, ro[g & 3], g >> 2);)
+    GEMM_XA(_Pragma("unroll") for (int g = 0; g < 8; g++) gemm_load_a1(a1.c[g], Xh + 1024, ro[g & 3], g >> 2);)
     half8_t b0[NF], b1[NF];
+#ifdef GEMM_X_NO_B
+#pragma unroll
+    for (int j = 0; j < NF; j++) b1[j] = half8_t{1, 1, 1, 1, 1, 1, 1, 1};
+#endif
     __syncthreads();  // R
     __syncthreads();  // stage 0 written
 #pragma unroll
-    for (int j = 0; j < NF; j++) b0[j] = *reinterpret_cast<const half8_t *>(smem + b_off + j * 16 * GBSTRIDE);
+    for (int j = 0; j < NF; j++) GEMM_LDB(b0[j], smem + b_off + j * 16 * GBSTRIDE);
 
-    // One stage: AC holds this stage's A fragments (requested a stage ago), AN receives the next.
-    // LAST drops what prepares a following stage.  cur / nxt are the LDS offsets of this stage's and
-    // the next stage's B buffers.
+    // One stage = eight groups of NF matrix instructions; group g multiplies A fragment g (rows
+    // (g % 4) * 16 .., k-half g / 4) of AC with the B fragments of that k-half, then requests the same
+    // fragment of the stage after next into the registers it has just consumed.  The requests are spread
+    // over the stage so that the four waves never queue more than the memory pipe takes without blocking
+    // the issue of the matrix instructions; a fragment is needed sixteen groups after its request, with
+    // fifteen younger requests outstanding.
+    // The B reads are spread the same way: the second k-half of this stage during groups 0..2, the
+    // first k-half of the next stage (after the barrier that publishes it) during groups 4..6.
+    // cur / nxt are the LDS offsets of this stage's and the next stage's B buffers.
     int cur = b_off, nxt = b_off + GB_HALFS;
-#define GEMM_STAGE(S, AC, AN, LAST)                                                                        \
+    constexpr int BPG = (NF + 2) / 3;  // B fragment reads per group
+#define GEMM_GROUP(G, AC, BV)                                                                              \
     {                                                                                                      \
-        GEMM_XA(if (!(LAST)) gemm_load_a(AN, Xh + ((S) + 1) * 1024, ro);)                                    \
-        if (LAST)                                                                                          \
-            GEMM_WAIT_A(0, AC);                                                                            \
-        else                                                                                               \
-            GEMM_WAIT_A(8, AC);                                                                            \
-        _Pragma("unroll") for (int j = 0; j < NF; j++)                                                     \
-            b1[j] = *reinterpret_cast<const half8_t *>(smem + cur + j * 16 * GBSTRIDE + 32);               \
-        __builtin_amdgcn_sched_barrier(0); /* keep the fragment reads ahead of the matrix instructions */  \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) _Pragma("unroll") for (int j = 0; j < NF; j++)       \
-            acc[i][j] = GEMM_MFMA(__builtin_bit_cast(half8_t, (AC).c[i]), b0[j], acc[i][j]);               \
+        GEMM_XA(asm volatile("s_waitcnt vmcnt(15)" : "+v"((AC).c[G])::"memory");)                          \
         __builtin_amdgcn_sched_barrier(0);                                                                 \
+        _Pragma("unroll") for (int j = 0; j < NF; j++) acc[(G) & 3][j] =                                   \
+            GEMM_MFMA(__builtin_bit_cast(half8_t, (AC).c[G]), BV[j], acc[(G) & 3][j]);                     \
+        __builtin_amdgcn_sched_barrier(0);                                                                 \
+        GEMM_XA(gemm_load_a1((AC).c[G], xs_next, ro[(G) & 3], (G) >> 2);)                                  \
+    }
+#define GEMM_BREADS(G3, DST, OFF)                                                                          \
+    _Pragma("unroll") for (int j = (G3) * BPG; j < NF && j < ((G3) + 1) * BPG; j++)                        \
+        GEMM_LDB(DST[j], smem + (OFF) + j * 16 * GBSTRIDE);
+#define GEMM_STAGE(S, AC, LAST)                                                                            \
+    {                                                                                                      \
+        const _Float16 *xs_next = Xh + min((S) + 2, nslots - 1) * 1024;                                    \
+        GEMM_BREADS(0, b1, cur + 32) GEMM_GROUP(0, AC, b0)                                                 \
+        GEMM_BREADS(1, b1, cur + 32) GEMM_GROUP(1, AC, b0)                                                 \
+        GEMM_BREADS(2, b1, cur + 32) GEMM_GROUP(2, AC, b0)                                                 \
+        GEMM_GROUP(3, AC, b0)                                                                              \
         if (!(LAST)) {                                                                                     \
             __syncthreads(); /* stage S+1 written */                                                       \
-            _Pragma("unroll") for (int j = 0; j < NF; j++)                                                 \
-                b0[j] = *reinterpret_cast<const half8_t *>(smem + nxt + j * 16 * GBSTRIDE);                \
+            GEMM_BREADS(0, b0, nxt)                                                                        \
         }                                                                                                  \
-        __builtin_amdgcn_sched_barrier(0);                                                                 \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) _Pragma("unroll") for (int j = 0; j < NF; j++)       \
-            acc[i][j] = GEMM_MFMA(__builtin_bit_cast(half8_t, (AC).c[4 + i]), b1[j], acc[i][j]);           \
+        GEMM_GROUP(4, AC, b1)                                                                              \
+        if (!(LAST)) { GEMM_BREADS(1, b0, nxt) }                                                           \
+        GEMM_GROUP(5, AC, b1)                                                                              \
+        if (!(LAST)) { GEMM_BREADS(2, b0, nxt) }                                                           \
+        GEMM_GROUP(6, AC, b1)                                                                              \
+        GEMM_GROUP(7, AC, b1)                                                                              \
         GEMM_XKEEP                                                                                         \
-        __builtin_amdgcn_sched_barrier(0);                                                                 \
         cur = nxt;                                                                                         \
         nxt = (nxt == b_off + (GNBUF - 1) * GB_HALFS) ? b_off : nxt + GB_HALFS;                            \
     }
     int s = 0;
     for (; s < nslots - 2; s += 2) {
-        GEMM_STAGE(s, a0, a1, false)
-        GEMM_STAGE(s + 1, a1, a0, false)
+        GEMM_STAGE(s, a0, false)
+        GEMM_STAGE(s + 1, a1, false)
     }
-    GEMM_STAGE(s, a0, a1, false)
-    GEMM_STAGE(s + 1, a1, a0, true)
+    GEMM_STAGE(s, a0, false)
+    GEMM_STAGE(s + 1, a1, true)
 #undef GEMM_STAGE
-
-    // every A request has been waited for: the last stage drained the counter
+#undef GEMM_GROUP
+#undef GEMM_BREADS
+    // the last two stages requested the last stage's fragments again (never used): drain before the registers die
+    GEMM_XA(GEMM_DRAIN_A(a0); GEMM_DRAIN_A(a1);)
 
     // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e
 #pragma unroll
@@ -454,7 +484,11 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + e;
+#ifdef GEMM_X_NO_STORE
+                if (m < M && n < N && acc[i][j][e] == 1234.5f) Y[(size_t)m * N + n] = acc[i][j][e];
+#else
                 if (m < M && n < N) Y[(size_t)m * N + n] = acc[i][j][e];
+#endif
             }
         }
 }
