@@ -321,26 +321,27 @@ __global__ __launch_bounds__(256) void gemv_q4_0_generic(const uint16_t *__restr
 constexpr int GG_MAX = 8;
 constexpr int GG_MAX_SLOTS = kChunkSlots;  // K <= 12288: one LDS pass
 
-struct gg_item {
-    const uint8_t *W;
-    const uint8_t *W2;      // up matrix of a SwiGLU pair, or null
-    float *dst;
-    const float *residual;  // or null
-    const float *x;
-    const float *norm_w;    // RMSNorm weight or null
-    float eps;
-    int32_t N;
-    int32_t nslots;
-    int32_t groups;  // row groups a wave works through, one after the other: amortises the preparation when N is large
-};
+// Kernel arguments, one array per field.  What a workgroup needs before it can request memory (matrix,
+// activations, shape) is fetched for all GG_MAX products at once and picked with scalar selects, so a
+// workgroup waits for one scalar load round trip, not for one per level of indexing.
 struct gg_args {
-    int32_t blk0[GG_MAX];  // first block of each matrix; unused entries hold INT_MAX
-    gg_item item[GG_MAX];
+    int32_t blk0[GG_MAX];         // first block of each matrix; unused entries hold INT_MAX
+    const uint8_t *W[GG_MAX];
+    const uint8_t *W2[GG_MAX];    // up matrix of a SwiGLU pair, or null
+    const float *x[GG_MAX];
+    int32_t N[GG_MAX];
+    int32_t nslots[GG_MAX];
+    int32_t groups[GG_MAX];       // row groups a wave works through, one after the other
+    const float *norm_w[GG_MAX];  // RMSNorm weight or null
+    float *dst[GG_MAX];
+    const float *residual[GG_MAX];  // or null
+    float eps[GG_MAX];
 };
 
 // A wave owns R slots per lane: R rows, or R / 2 rows of a gate / up pair; a workgroup WAVES times that.
 // PG: activation groups (8 values) one thread prepares at most; NORM: the vector is normalised first.
-template <int L, int R, int WAVES, int PG, int OCC, bool NORM>
+// MAXI: products the selects look at (4 keeps all of their operands in scalar registers at once).
+template <int L, int R, int WAVES, int PG, int OCC, bool NORM, int MAXI>
 __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     __shared__ float red[WAVES];
@@ -350,18 +351,44 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     const int wave = threadIdx.x >> 6;
     GH_TSTAMP(0);
 
-    int ii = 0;
+    // Every product's fields are fetched before any is chosen (the empty asm makes each an opaque value; left
+    // alone, the compiler turns a select of two arguments into a second, dependent load from a selected address).
+    int32_t k_blk0[MAXI], k_N[MAXI], k_ns[MAXI], k_groups[MAXI];
+    uint64_t k_W[MAXI], k_W2[MAXI], k_x[MAXI];  // pointers as bits: an address that has been through an asm is
+                                                // no longer known to be global memory and is cast back below
 #pragma unroll
-    for (int k = 1; k < GG_MAX; k++)
-        if ((int)blockIdx.x >= a.blk0[k]) ii = k;
-    const gg_item &it = a.item[ii];
-    const uint8_t *const W = it.W, *const W2 = it.W2;
+    for (int k = 0; k < MAXI; k++) {
+        k_blk0[k] = a.blk0[k], k_N[k] = a.N[k], k_ns[k] = a.nslots[k], k_groups[k] = a.groups[k];
+        k_W[k] = (uint64_t)a.W[k], k_W2[k] = (uint64_t)a.W2[k], k_x[k] = (uint64_t)a.x[k];
+    }
+#pragma unroll
+    for (int k = 0; k < MAXI; k++) {
+        asm volatile("" : "+s"(k_blk0[k]));
+        asm volatile("" : "+s"(k_N[k]));
+        asm volatile("" : "+s"(k_ns[k]));
+        asm volatile("" : "+s"(k_groups[k]));
+        asm volatile("" : "+s"(k_W[k]));
+        asm volatile("" : "+s"(k_W2[k]));
+        asm volatile("" : "+s"(k_x[k]));
+    }
+    int ii = 0, first_blk = 0;
+    uint64_t W_bits = k_W[0], W2_bits = k_W2[0], x_bits = k_x[0];
+    int N = k_N[0], ns = k_ns[0], groups = k_groups[0];
+#pragma unroll
+    for (int k = 1; k < MAXI; k++) {
+        const bool ge = (int)blockIdx.x >= k_blk0[k];
+        ii = ge ? k : ii, first_blk = ge ? k_blk0[k] : first_blk;
+        W_bits = ge ? k_W[k] : W_bits, W2_bits = ge ? k_W2[k] : W2_bits, x_bits = ge ? k_x[k] : x_bits;
+        N = ge ? k_N[k] : N, ns = ge ? k_ns[k] : ns, groups = ge ? k_groups[k] : groups;
+    }
+    typedef const __attribute__((address_space(1))) uint8_t *global_bytes;
+    typedef const __attribute__((address_space(1))) float *global_floats;
+    const uint8_t *const W = (const uint8_t *)(global_bytes)W_bits, *const W2 = (const uint8_t *)(global_bytes)W2_bits;
+    const float *const xg = (const float *)(global_floats)x_bits;
     const bool dual = W2 != nullptr;
-    const int N = it.N, ns = it.nslots;
     const int rw = dual ? R / 2 : R;  // rows per wave and group
-    const int groups = it.groups;
     // group g of the workgroup's waves covers WAVES * rw consecutive rows: neighbouring waves read neighbouring rows
-    const int wg_row0 = ((int)blockIdx.x - a.blk0[ii]) * (WAVES * rw * groups);
+    const int wg_row0 = ((int)blockIdx.x - first_blk) * (WAVES * rw * groups);
     int row0 = wg_row0 + wave * rw;
     const size_t row_bytes = (size_t)ns * sizeof(q4_slot);
     GH_TSTAMP(1);
@@ -374,8 +401,9 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     // are requested first and the first weights right behind them: the preparation then runs while the weights
     // are in flight.
     q4_slot q0[R];
+    uint64_t dst_bits, res_bits;
     {
-        const float *xg = it.x, *wg = it.norm_w;
+        const float *wg = NORM ? a.norm_w[ii] : nullptr;
         float2 v[PG][4], nw[NORM ? PG : 1][4];
 #pragma unroll
         for (int p = 0; p < PG; p++) {
@@ -406,6 +434,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             }
         }
         GH_TSTAMP(2);
+        // Where the results go, fetched now (indexed argument loads) so that nothing waits for them at the end.
+        dst_bits = (uint64_t)a.dst[ii], res_bits = (uint64_t)a.residual[ii];
+        asm volatile("" : "+s"(dst_bits));
+        asm volatile("" : "+s"(res_bits));
         if (NORM) {
             float ss = 0.0f;
 #pragma unroll
@@ -420,7 +452,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             float tot = 0.0f;
 #pragma unroll
             for (int w = 0; w < WAVES; w++) tot += red[w];
-            const float inv = rsqrtf(tot / (float)(ns * 64) + it.eps);
+            const float inv = rsqrtf(tot / (float)(ns * 64) + a.eps[ii]);
 #pragma unroll
             for (int p = 0; p < PG; p++)
 #pragma unroll
@@ -515,8 +547,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             }
         }
         if (lane < rw && row0 + lane < N) {
-            if (it.residual) out += it.residual[row0 + lane];
-            it.dst[row0 + lane] = out;
+            typedef __attribute__((address_space(1))) float *global_out;
+            const float *res = (const float *)(global_floats)res_bits;
+            if (res) out += res[row0 + lane];
+            ((float *)(global_out)dst_bits)[row0 + lane] = out;
         }
 #pragma unroll
         for (int j = 0; j < R; j++) acc[j] = 0.0f;
@@ -551,7 +585,7 @@ void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst
 }
 
 // Host side of the group kernel: checks, the block range of every matrix, launch.
-template <int L, int R, int WAVES, int OCC>
+template <int L, int R, int WAVES, int OCC, int MAXI>
 void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, int max_slots, bool norm) {
     const dim3 grid(blocks), block(WAVES * 64);
     const size_t lds = (size_t)max_slots * slot_lds<L>::dwords * sizeof(uint32_t);
@@ -559,15 +593,24 @@ void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, in
     constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
     if (max_slots <= 64) {
         if (norm)
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true>), grid, block, lds, ctx->stream, a);
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true, MAXI>), grid, block, lds, ctx->stream, a);
         else
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, false>), grid, block, lds, ctx->stream, a);
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, false, MAXI>), grid, block, lds, ctx->stream, a);
     } else {
         if (norm)  // the normalising preparation of a long vector needs more than 64 registers
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, (OCC > 4 ? 4 : OCC), true>), grid, block, lds, ctx->stream, a);
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, (OCC > 4 ? 4 : OCC), true, MAXI>), grid, block, lds,
+                               ctx->stream, a);
         else
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, false>), grid, block, lds, ctx->stream, a);
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, false, MAXI>), grid, block, lds, ctx->stream, a);
     }
+}
+
+template <int L, int R, int WAVES, int OCC>
+void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, int n_items, unsigned blocks, int max_slots, bool norm) {
+    if (n_items <= 4)
+        launch_group_cfg<L, R, WAVES, OCC, 4>(ctx, a, blocks, max_slots, norm);
+    else
+        launch_group_cfg<L, R, WAVES, OCC, GG_MAX>(ctx, a, blocks, max_slots, norm);
 }
 
 int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what) {
@@ -590,14 +633,13 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
         if (i == 0) norm = s.norm_weight != nullptr;
         GH_REQUIRE(ctx, (s.norm_weight != nullptr) == norm, GALOIS_HIP_E_UNSUPPORTED,
                    "gemv group: either every product of a call normalises its activations or none does");
-        gg_item &d = a.item[i];
-        d.W = (const uint8_t *)s.vx, d.W2 = (const uint8_t *)s.vx_up, d.dst = s.dst, d.residual = s.residual;
-        d.x = s.y, d.norm_w = s.norm_weight, d.eps = s.norm_eps, d.N = s.nrows, d.nslots = s.ncols / 64;
-        if (d.nslots > max_slots) max_slots = d.nslots;
+        a.W[i] = (const uint8_t *)s.vx, a.W2[i] = (const uint8_t *)s.vx_up, a.dst[i] = s.dst, a.residual[i] = s.residual;
+        a.x[i] = s.y, a.norm_w[i] = s.norm_weight, a.eps[i] = s.norm_eps, a.N[i] = s.nrows, a.nslots[i] = s.ncols / 64;
+        if (a.nslots[i] > max_slots) max_slots = a.nslots[i];
         rows += (int64_t)s.nrows * (s.vx_up ? 2 : 1);
     }
     // Workgroup shape by rows per CU, as for the one-product kernel: few rows -> 16 waves x 1 slot so every SIMD has
-    // work; more rows -> 8 waves x 2 slots, four workgroups resident per CU.  A gate / up pair needs 2 slots per lane.
+    // work; more rows -> 8 waves x 2 slots, three workgroups resident per CU.  A gate / up pair needs 2 slots per lane.
     bool any_dual = false;
     for (int i = 0; i < n_items; i++) any_dual |= items[i].vx_up != nullptr;
     int cfg = ctx->gemv_config;
@@ -611,7 +653,7 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
         int groups = ctx->gemv_units_per_wave;
         if (groups <= 0) groups = 1;
         groups = groups < 1 ? 1 : (groups > 4 ? 4 : groups);
-        a.item[i].groups = groups;
+        a.groups[i] = groups;
         const int64_t rows_per_wg = (items[i].vx_up ? slots_per_wg / 2 : slots_per_wg) * groups;
         a.blk0[i] = (int32_t)blocks;
         blocks += (items[i].nrows + rows_per_wg - 1) / rows_per_wg;
@@ -619,11 +661,11 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     }
     GH_BIND(ctx);
     if (cfg == 1)
-        launch_group_cfg<5, 1, 16, 4>(ctx, a, (unsigned)blocks, max_slots, norm);
+        launch_group_cfg<5, 1, 16, 4>(ctx, a, n_items, (unsigned)blocks, max_slots, norm);
     else if (cfg == 7)
-        launch_group_cfg<5, 2, 8, 8>(ctx, a, (unsigned)blocks, max_slots, norm);
+        launch_group_cfg<5, 2, 8, 8>(ctx, a, n_items, (unsigned)blocks, max_slots, norm);
     else
-        launch_group_cfg<5, 2, 8, 4>(ctx, a, (unsigned)blocks, max_slots, norm);
+        launch_group_cfg<5, 2, 8, 6>(ctx, a, n_items, (unsigned)blocks, max_slots, norm);
     GH_LAUNCH_CHECK(ctx, what);
 }
 
