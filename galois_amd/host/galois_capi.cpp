@@ -3,17 +3,22 @@
 #include <string>
 
 #include "galois.hpp"
+#include "gguf.hpp"
 #include "llama.hpp"
 
 using namespace galois;
 
 static thread_local std::string g_last_error;
+static thread_local int g_last_kind = 0;
 static int fail(const GResult &r) {
     g_last_error = r.msg;
+    g_last_kind = (int)r.kind;
     return (int)r.kind;
 }
 
 extern "C" {
+// GError kind of the failure galois_host_last_error() describes (for functions that return a handle)
+int galois_host_last_error_kind() { return g_last_kind; }
 
 const char *galois_host_last_error() { return g_last_error.c_str(); }
 
@@ -203,6 +208,97 @@ int galois_host_llama_time_steps(void *m, void *dev, int32_t token, int32_t n_pa
     galois_hip_event_destroy(ctx, e1);
     if (!r.ok()) return fail(r);
     return st ? fail(GError{GError::DeviceError, galois_hip_last_error(ctx)}) : 0;
+}
+
+// ---- GGUF model files -----------------------------------------------------------------------------
+// Functions returning a handle return null on failure, functions returning int the GError kind (0 = ok);
+// galois_host_last_error() then holds the message.
+void *galois_host_gguf_open(const char *path) {
+    std::unique_ptr<GgufFile> f;
+    GResult r = GgufFile::open(path, &f);
+    if (!r.ok()) {
+        fail(r);
+        return nullptr;
+    }
+    return f.release();
+}
+void galois_host_gguf_close(void *f) { delete (GgufFile *)f; }
+uint32_t galois_host_gguf_version(void *f) { return ((GgufFile *)f)->version(); }
+size_t galois_host_gguf_alignment(void *f) { return ((GgufFile *)f)->alignment(); }
+size_t galois_host_gguf_data_start(void *f) { return ((GgufFile *)f)->data_start(); }
+size_t galois_host_gguf_n_tensors(void *f) { return ((GgufFile *)f)->tensors().size(); }
+size_t galois_host_gguf_n_kv(void *f) { return ((GgufFile *)f)->metadata().size(); }
+// name (borrowed, valid while the file is open), n_dims, shape[4], ggml type id, offset, nbytes, supported
+const char *galois_host_gguf_tensor_info(void *f, size_t idx, size_t *n_dims, size_t *shape, uint32_t *ggml_type,
+                                         uint64_t *offset, size_t *nbytes, int *supported) {
+    const auto &ts = ((GgufFile *)f)->tensors();
+    if (idx >= ts.size()) {
+        fail(GError{GError::Unexpected, "gguf: tensor index out of range"});
+        return nullptr;
+    }
+    const GgufTensorInfo &t = ts[idx];
+    *n_dims = t.n_dims;
+    for (int d = 0; d < 4; d++) shape[d] = t.shape[d];
+    *ggml_type = t.ggml_type, *offset = t.offset, *nbytes = t.nbytes, *supported = t.supported ? 1 : 0;
+    return t.name.c_str();
+}
+int galois_host_gguf_get_uint(void *f, const char *key, uint64_t *out) { return ((GgufFile *)f)->get_uint(key, out) ? 1 : 0; }
+int galois_host_gguf_get_float(void *f, const char *key, double *out) { return ((GgufFile *)f)->get_float(key, out) ? 1 : 0; }
+// copies at most cap - 1 bytes and a terminator; returns the string's length, or -1 when the key is no string
+long galois_host_gguf_get_string(void *f, const char *key, char *buf, size_t cap) {
+    std::string s;
+    if (!((GgufFile *)f)->get_string(key, &s)) return -1;
+    if (cap > 0) {
+        const size_t n = s.size() < cap - 1 ? s.size() : cap - 1;
+        memcpy(buf, s.data(), n);
+        buf[n] = 0;
+    }
+    return (long)s.size();
+}
+// number of elements of a string array and the length of element i (copied like get_string); -1 = no such array
+long galois_host_gguf_string_array(void *f, const char *key, size_t i, char *buf, size_t cap) {
+    std::vector<std::string> v;
+    GResult r = ((GgufFile *)f)->get_string_array(key, &v);
+    if (!r.ok()) {
+        fail(r);
+        return -1;
+    }
+    if (!buf) return (long)v.size();
+    if (i >= v.size()) return -1;
+    const size_t n = cap == 0 ? 0 : (v[i].size() < cap - 1 ? v[i].size() : cap - 1);
+    if (cap > 0) {
+        memcpy(buf, v[i].data(), n);
+        buf[n] = 0;
+    }
+    return (long)v[i].size();
+}
+void *galois_host_gguf_load_tensor(void *f, const char *name, void *dev) {
+    Tensor *t = new Tensor();
+    GResult r = ((GgufFile *)f)->load_tensor(name, *(Device *)dev, t);
+    if (!r.ok()) {
+        delete t;
+        fail(r);
+        return nullptr;
+    }
+    return t;
+}
+// hp[6] = n_vocab, n_embd, n_head, n_layer, n_ff, n_ctx; fp[3] = rms_eps, freq_base, freq_scale
+int galois_host_gguf_llama_hparams(void *f, size_t n_ctx_max, size_t *hp, float *fp) {
+    LlamaHParams h;
+    GResult r = llama_hparams_from_gguf(*(GgufFile *)f, n_ctx_max, &h);
+    if (!r.ok()) return fail(r);
+    hp[0] = h.n_vocab, hp[1] = h.n_embd, hp[2] = h.n_head, hp[3] = h.n_layer, hp[4] = h.n_ff, hp[5] = h.n_ctx;
+    fp[0] = h.rms_eps, fp[1] = h.freq_base, fp[2] = h.freq_scale;
+    return 0;
+}
+void *galois_host_llama_from_gguf(void *f, void *dev, size_t n_ctx_max) {
+    std::unique_ptr<LlamaDecoder> m;
+    GResult r = llama_from_gguf(*(GgufFile *)f, *(Device *)dev, n_ctx_max, &m);
+    if (!r.ok()) {
+        fail(r);
+        return nullptr;
+    }
+    return m.release();
 }
 
 }  // extern "C"

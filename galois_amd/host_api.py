@@ -34,6 +34,7 @@ def lib():
         L = C.CDLL(LIB_PATH)
         vp, sz = C.c_void_p, C.c_size_t
         L.galois_host_last_error.restype = C.c_char_p
+        L.galois_host_last_error_kind.restype = C.c_int
         for name, res, args in (
                 ("galois_host_device_new", vp, [C.c_int]), ("galois_host_device_cpu", vp, []),
                 ("galois_host_device_free", None, [vp]),
@@ -60,14 +61,31 @@ def lib():
                 ("galois_host_llama_replay", C.c_int, [vp]),
                 ("galois_host_llama_time_replays", C.c_int, [vp, vp, C.c_int, C.POINTER(C.c_float)]),
                 ("galois_host_llama_time_steps", C.c_int, [vp, vp, C.c_int32, C.c_int32, C.c_int, C.c_int,
-                                                           C.POINTER(C.c_float)])):
+                                                           C.POINTER(C.c_float)]),
+                ("galois_host_gguf_open", vp, [C.c_char_p]), ("galois_host_gguf_close", None, [vp]),
+                ("galois_host_gguf_version", C.c_uint32, [vp]), ("galois_host_gguf_alignment", sz, [vp]),
+                ("galois_host_gguf_data_start", sz, [vp]), ("galois_host_gguf_n_tensors", sz, [vp]),
+                ("galois_host_gguf_n_kv", sz, [vp]),
+                ("galois_host_gguf_tensor_info", C.c_char_p, [vp, sz, C.POINTER(sz), C.POINTER(sz),
+                                                              C.POINTER(C.c_uint32), C.POINTER(C.c_uint64),
+                                                              C.POINTER(sz), C.POINTER(C.c_int)]),
+                ("galois_host_gguf_get_uint", C.c_int, [vp, C.c_char_p, C.POINTER(C.c_uint64)]),
+                ("galois_host_gguf_get_float", C.c_int, [vp, C.c_char_p, C.POINTER(C.c_double)]),
+                ("galois_host_gguf_get_string", C.c_long, [vp, C.c_char_p, C.c_char_p, sz]),
+                ("galois_host_gguf_string_array", C.c_long, [vp, C.c_char_p, sz, C.c_char_p, sz]),
+                ("galois_host_gguf_load_tensor", vp, [vp, C.c_char_p, vp]),
+                ("galois_host_gguf_llama_hparams", C.c_int, [vp, sz, C.POINTER(sz), C.POINTER(C.c_float)]),
+                ("galois_host_llama_from_gguf", vp, [vp, vp, sz])):
             fn = getattr(L, name)
             fn.restype, fn.argtypes = res, args
         _lib = L
     return _lib
 
 
-def _raise(kind=4):
+def _raise(kind=None):
+    """Raises the library's last error; kind None = the kind the library recorded with it."""
+    if kind is None:
+        kind = lib().galois_host_last_error_kind() or 4
     raise GError(kind, lib().galois_host_last_error().decode())
 
 
@@ -207,14 +225,24 @@ class LlamaDecoder:
     """One-token decode step of a LLaMA-architecture model issued as galois ops (galois_amd/host/llama.hpp)."""
 
     def __init__(self, device, n_vocab=32000, n_embd=4096, n_head=32, n_layer=32, n_ff=11008, n_ctx=2048,
-                 rms_eps=1e-6, freq_base=10000.0):
+                 rms_eps=1e-6, freq_base=10000.0, _handle=None):
         self.device = device
         self.hp = dict(n_vocab=n_vocab, n_embd=n_embd, n_head=n_head, n_layer=n_layer, n_ff=n_ff, n_ctx=n_ctx,
                        rms_eps=rms_eps, freq_base=freq_base)
-        self.h = lib().galois_host_llama_new(device.h, n_vocab, n_embd, n_head, n_layer, n_ff, n_ctx, rms_eps,
-                                             freq_base)
+        self.h = _handle or lib().galois_host_llama_new(device.h, n_vocab, n_embd, n_head, n_layer, n_ff, n_ctx,
+                                                        rms_eps, freq_base)
         if not self.h:
             _raise(3)
+
+    @staticmethod
+    def from_gguf(gguf, device, n_ctx_max=2048):
+        """A decoder with the hyper-parameters and the weights of a GGUF file (``GgufFile``)."""
+        hp = gguf.llama_hparams(n_ctx_max)
+        h = lib().galois_host_llama_from_gguf(gguf.h, device.h, n_ctx_max)
+        if not h:
+            _raise()
+        hp.pop("freq_scale")
+        return LlamaDecoder(device, _handle=h, **hp)
 
     def close(self):
         if self.h:
@@ -263,3 +291,92 @@ class LlamaDecoder:
         ms = C.c_float()
         _call(lib().galois_host_llama_time_steps(self.h, self.device.h, token, n_past, int(fused), n, C.byref(ms)))
         return ms.value
+
+
+class GgufFile:
+    """A memory-mapped GGUF model file (galois_amd/host/gguf.hpp): metadata, tensor table, tensors as ``Tensor``."""
+
+    def __init__(self, path):
+        self.h = lib().galois_host_gguf_open(os.fsencode(path))
+        if not self.h:
+            _raise()
+
+    def close(self):
+        if self.h:
+            lib().galois_host_gguf_close(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @property
+    def version(self):
+        return lib().galois_host_gguf_version(self.h)
+
+    @property
+    def alignment(self):
+        return lib().galois_host_gguf_alignment(self.h)
+
+    @property
+    def data_start(self):
+        return lib().galois_host_gguf_data_start(self.h)
+
+    @property
+    def n_kv(self):
+        return lib().galois_host_gguf_n_kv(self.h)
+
+    def tensors(self):
+        """List of dicts: name, shape (ne0 first), ggml_type, offset, nbytes, supported."""
+        out = []
+        for i in range(lib().galois_host_gguf_n_tensors(self.h)):
+            nd, shape = C.c_size_t(), (C.c_size_t * 4)()
+            ty, off, nb, sup = C.c_uint32(), C.c_uint64(), C.c_size_t(), C.c_int()
+            name = lib().galois_host_gguf_tensor_info(self.h, i, C.byref(nd), shape, C.byref(ty), C.byref(off),
+                                                      C.byref(nb), C.byref(sup))
+            out.append({"name": name.decode(), "shape": tuple(shape[:nd.value]), "ggml_type": ty.value,
+                        "offset": off.value, "nbytes": nb.value, "supported": bool(sup.value)})
+        return out
+
+    def get_uint(self, key):
+        v = C.c_uint64()
+        return v.value if lib().galois_host_gguf_get_uint(self.h, key.encode(), C.byref(v)) else None
+
+    def get_float(self, key):
+        v = C.c_double()
+        return v.value if lib().galois_host_gguf_get_float(self.h, key.encode(), C.byref(v)) else None
+
+    def get_string(self, key):
+        n = lib().galois_host_gguf_get_string(self.h, key.encode(), None, 0)
+        if n < 0:
+            return None
+        buf = C.create_string_buffer(n + 1)
+        lib().galois_host_gguf_get_string(self.h, key.encode(), buf, n + 1)
+        return buf.raw[:n].decode("utf-8", "replace")
+
+    def get_string_array(self, key):
+        n = lib().galois_host_gguf_string_array(self.h, key.encode(), 0, None, 0)
+        if n < 0:
+            return None
+        out = []
+        buf = C.create_string_buffer(1 << 16)
+        for i in range(n):
+            m = lib().galois_host_gguf_string_array(self.h, key.encode(), i, buf, len(buf))
+            out.append(buf.raw[:min(m, len(buf) - 1)].decode("utf-8", "replace"))
+        return out
+
+    def load_tensor(self, name, device):
+        """``Tensor::from_raw`` on the tensor's bytes (F32, F16 and Q4_0 tensors)."""
+        info = next((t for t in self.tensors() if t["name"] == name), None)
+        h = lib().galois_host_gguf_load_tensor(self.h, name.encode(), device.h)
+        if not h:
+            _raise()
+        return Tensor(h, info["shape"], info["ggml_type"])
+
+    def llama_hparams(self, n_ctx_max=2048):
+        hp, fp = (C.c_size_t * 6)(), (C.c_float * 3)()
+        _call(lib().galois_host_gguf_llama_hparams(self.h, n_ctx_max, hp, fp))
+        return dict(n_vocab=hp[0], n_embd=hp[1], n_head=hp[2], n_layer=hp[3], n_ff=hp[4], n_ctx=hp[5],
+                    rms_eps=fp[0], freq_base=fp[1], freq_scale=fp[2])
