@@ -3,16 +3,16 @@
 // In galois's op vocabulary a decode step's attention is rope_custom(q), rope_custom(k), cpy(k -> cache row),
 // cpy(v -> cache row), matmul(K^T, q), scale, soft_max, matmul(V, p) (launchers src/cuda.rs:1257-1356, 1382-1595,
 // 698-782, 1597-1663).  Issued one by one these are nine launches that read the 64 MB of one layer's cache at
-// a third of the HBM rate, most of the time being launch gaps.  Here the same arithmetic runs in two launches:
+// a third of the HBM rate, most of the time being launch gaps.  Here the same arithmetic runs in one launch:
 //
 //   attn_decode_partial: a workgroup owns 128 consecutive keys of one head.  It rotates its head's q (every
 //     workgroup of the head does, it is 128 floats), and the workgroup that owns position n_past also rotates
 //     the new k and writes k and v into row n_past of the caches.  Scores = scale * (k . q) go to LDS; the
 //     workgroup takes their maximum m, p = exp(score - m), the sum of p and the partial output sum p * v, and
-//     writes (m, sum, partial output) to the context's scratch block;
-//   attn_decode_combine: per head, rescales the partials to the global maximum, adds them in split order and
-//     divides by the total: out = softmax(scores) . V exactly as the three separate ops define it, up to the
-//     order of the f32 additions.
+//     writes (m, sum, partial output) to the context's scratch block, then counts itself on the head's counter;
+//   the workgroup that counts a head's last split rescales the head's partials to the global maximum, adds them
+//     in split order and divides by the total: out = softmax(scores) . V exactly as the three separate ops
+//     define it, up to the order of the f32 additions (the result does not depend on which workgroup merges).
 //
 // A lane owns 4 consecutive floats of a head; head_dim / 4 lanes cover one key, so a wave-load of 16 bytes per
 // lane reads 64 / (head_dim / 4) whole cache rows of the head (512 contiguous bytes each for head_dim 128).
@@ -68,12 +68,66 @@ struct at_rot {
     }
 };
 
+// Device-coherent accesses to the split records: relaxed atomics of device scope are plain loads and stores that
+// bypass the caches private to a CU or an XCD, so a record written on one XCD is read correctly on another
+// without any cache being flushed.
+__device__ __forceinline__ void at_store(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float at_load(const float *p) {
+    return __hip_atomic_load(const_cast<float *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Merge of a head's splits, run by the workgroup that finishes the head's last split: thread d < D owns output
+// element d.  The split maxima and sums are fetched by S threads at once and the weights exp(m_s - M) shared
+// through LDS; the partial outputs are then read eight splits at a time.
+constexpr int AT_MAX_SPLITS = 1024;
+__device__ __forceinline__ void at_combine(const float *rec, float *__restrict__ out_h, int D, int S, float *w,
+                                           float (*red)[AT_THREADS / 64]) {
+    constexpr int WAVES = AT_THREADS / 64;
+    const int d = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mx = -__builtin_inff();
+    for (int s = d; s < S; s += AT_THREADS) {
+        const float ms = at_load(rec + (size_t)s * (D + 4));
+        w[s] = ms;
+        mx = fmaxf(mx, ms);
+    }
+    mx = at_wave_max(mx);
+    if (lane == 0) red[0][wave] = mx;
+    __syncthreads();
+    float M = red[0][0];
+#pragma unroll
+    for (int i = 1; i < WAVES; i++) M = fmaxf(M, red[0][i]);
+    float den = 0.0f;
+    for (int s = d; s < S; s += AT_THREADS) {
+        const float ws = expf(w[s] - M);
+        w[s] = ws;
+        den = __builtin_fmaf(ws, at_load(rec + (size_t)s * (D + 4) + 1), den);
+    }
+    den = at_wave_sum(den);
+    if (lane == 0) red[1][wave] = den;
+    __syncthreads();
+    den = red[1][0];
+#pragma unroll
+    for (int i = 1; i < WAVES; i++) den += red[1][i];
+    if (d < D) {
+        float num = 0.0f;
+        for (int s0 = 0; s0 < S; s0 += 8) {
+            float o[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) o[j] = at_load(rec + (size_t)min(s0 + j, S - 1) * (D + 4) + 4 + d);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (s0 + j < S) num = __builtin_fmaf(w[s0 + j], o[j], num);
+        }
+        out_h[d] = num / den;
+    }
+}
+
 // Record of one (head, split) in the scratch block: m, sum, 2 unused floats, then head_dim partial outputs.
 template <int LPR>
 __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *__restrict__ q, const float *__restrict__ k,
                                                                   const float *__restrict__ v, float *__restrict__ kc,
                                                                   float *__restrict__ vc, float *__restrict__ part,
-                                                                  float *__restrict__ out, int H, int L,
+                                                                  unsigned *__restrict__ done, float *__restrict__ out, int H, int L,
                                                                   const int32_t *__restrict__ pos, float freq_scale,
                                                                   float theta_scale, float scale) {
     constexpr int D = LPR * 4, RPL = 64 / LPR, WAVES = AT_THREADS / 64;
@@ -82,6 +136,9 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
     __shared__ float sc[AT_KEYS];
     __shared__ float4 ored[WAVES][LPR];
     __shared__ float sred[WAVES];
+    __shared__ float cw[AT_MAX_SPLITS];
+    __shared__ float cred[2][WAVES];
+    __shared__ unsigned last_flag;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane / LPR, kl = lane % LPR;
     const int h = blockIdx.y, s = blockIdx.x, S = gridDim.x;
@@ -180,52 +237,28 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
             const float inv = 1.0f / tot;
             *reinterpret_cast<float4 *>(out + (size_t)h * D + lane * 4) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
         } else {
+            // The record goes out as device-coherent stores (they bypass the XCD-local caches) and is waited for
+            // before the split is counted; a device-wide fence here would write back and invalidate the whole L2
+            // once per workgroup (measured: the kernel takes almost three times as long).
             float *rec = part + ((size_t)h * S + s) * (D + 4);
-            if (lane == 0) rec[0] = m, rec[1] = tot;
-            *reinterpret_cast<float4 *>(rec + 4 + lane * 4) = o;
+            if (lane == 0) at_store(rec, m), at_store(rec + 1, tot);
+            at_store(rec + 4 + lane * 4, o.x), at_store(rec + 5 + lane * 4, o.y);
+            at_store(rec + 6 + lane * 4, o.z), at_store(rec + 7 + lane * 4, o.w);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     }
-}
-
-// One workgroup per head, one thread per output element.  The split maxima and sums are fetched by S threads at
-// once and the weights exp(m_s - M) shared through LDS; the partial outputs are then read eight splits at a time.
-constexpr int AT_MAX_SPLITS = 1024;
-__global__ void attn_decode_combine(const float *__restrict__ part, float *__restrict__ out, int D, int S) {
-    __shared__ float w[AT_MAX_SPLITS];
-    __shared__ float red[2][2];
-    const int h = blockIdx.x, d = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int nwaves = blockDim.x >> 6;
-    const float *rec = part + (size_t)h * S * (D + 4);
-    float mx = -__builtin_inff();
-    for (int s = d; s < S; s += blockDim.x) {
-        const float2 ms = *reinterpret_cast<const float2 *>(rec + (size_t)s * (D + 4));
-        w[s] = ms.x;
-        mx = fmaxf(mx, ms.x);
-    }
-    mx = at_wave_max(mx);
-    if (lane == 0) red[0][wave] = mx;
+    if (S == 1) return;
+    // The workgroup that counts the head's last split merges all of them (no second launch).  The counter
+    // returns to zero for the next call.
     __syncthreads();
-    const float M = nwaves == 1 ? red[0][0] : fmaxf(red[0][0], red[0][1]);
-    float den = 0.0f;
-    for (int s = d; s < S; s += blockDim.x) {
-        const float ws = expf(w[s] - M);
-        w[s] = ws;
-        den = __builtin_fmaf(ws, rec[(size_t)s * (D + 4) + 1], den);
+    if (threadIdx.x == 0) {
+        const unsigned prev = atomicAdd(done + h, 1u);
+        last_flag = prev == (unsigned)(S - 1);
+        if (last_flag) done[h] = 0;
     }
-    den = at_wave_sum(den);
-    if (lane == 0) red[1][wave] = den;
     __syncthreads();
-    den = nwaves == 1 ? red[1][0] : red[1][0] + red[1][1];
-    float num = 0.0f;
-    for (int s0 = 0; s0 < S; s0 += 8) {
-        float o[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) o[j] = rec[(size_t)min(s0 + j, S - 1) * (D + 4) + 4 + d];
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-            if (s0 + j < S) num = __builtin_fmaf(w[s0 + j], o[j], num);
-    }
-    out[(size_t)h * D + d] = num / den;
+    if (!last_flag) return;
+    at_combine(part + (size_t)h * S * (D + 4), out + (size_t)h * D, D, S, cw, cred);
 }
 
 }  // namespace
@@ -244,20 +277,18 @@ extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *
                GALOIS_HIP_E_ALIGN, "attn_decode_f32: 16-byte aligned vectors and caches");
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
-    GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && (int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr),
+    GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && (int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr && ctx->attn_done != nullptr),
                GALOIS_HIP_E_UNSUPPORTED, "attn_decode_f32: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
                                          "results must fit the context's 4 MB scratch block");
     GH_BIND(ctx);
     float *part = (float *)ctx->scratch;
+    unsigned *done = ctx->attn_done;  // one counter per head, zero between calls
     const dim3 grid((unsigned)S, (unsigned)n_head), block(AT_THREADS);
     if (head_dim == 128)
-        hipLaunchKernelGGL(attn_decode_partial<32>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, out,
+        hipLaunchKernelGGL(attn_decode_partial<32>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done, out,
                            n_head, L, pos, freq_scale, theta_scale, scale);
     else
-        hipLaunchKernelGGL(attn_decode_partial<16>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, out,
+        hipLaunchKernelGGL(attn_decode_partial<16>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done, out,
                            n_head, L, pos, freq_scale, theta_scale, scale);
-    if (S > 1)
-        hipLaunchKernelGGL(attn_decode_combine, dim3((unsigned)n_head), dim3((unsigned)head_dim), 0, ctx->stream, part, out,
-                           head_dim, S);
     GH_LAUNCH_CHECK(ctx, "attn_decode_f32 launch");
 }

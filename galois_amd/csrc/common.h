@@ -15,13 +15,15 @@ struct galois_hip_ctx {
     int32_t gemv_units_per_wave;  // 0 = choose from the shape; GALOIS_HIP_GEMV_UNITS forces it (tuning)
     void *ws;         // workspace owned by the context (fp16 activations of the prefill matmul)
     size_t ws_bytes;
-    void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul
+    void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul, partial results of the decode attention
+    unsigned *attn_done;  // GH_ATTN_HEADS counters of the decode attention (splits finished per head), zero between calls
     bool capturing;   // between graph_begin_capture and graph_end_capture: nothing may allocate or block
     char last_error[256];
 };
 
 // galois_hip_ctx::scratch holds GH_PARTIAL_FLOATS floats of partial sums.
 constexpr int64_t GH_PARTIAL_FLOATS = 1 << 20;
+constexpr int64_t GH_ATTN_HEADS = 65536;
 
 struct galois_hip_event {
     hipEvent_t ev;

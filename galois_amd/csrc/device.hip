@@ -39,6 +39,7 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     ctx->ws = nullptr;
     ctx->ws_bytes = 0;
     ctx->scratch = nullptr;
+    ctx->attn_done = nullptr;
     ctx->capturing = false;
     const char *cfg = getenv("GALOIS_HIP_GEMV_CONFIG");
     ctx->gemv_config = cfg ? atoi(cfg) : 0;
@@ -52,9 +53,12 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     const size_t scratch_bytes = GH_PARTIAL_FLOATS * sizeof(float);
     e = hipMalloc(&ctx->scratch, scratch_bytes);
     if (e == hipSuccess) e = hipMemsetAsync(ctx->scratch, 0, scratch_bytes, ctx->stream);
+    if (e == hipSuccess) e = hipMalloc((void **)&ctx->attn_done, GH_ATTN_HEADS * sizeof(unsigned));
+    if (e == hipSuccess) e = hipMemsetAsync(ctx->attn_done, 0, GH_ATTN_HEADS * sizeof(unsigned), ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
         if (ctx->scratch) (void)hipFree(ctx->scratch);
+        if (ctx->attn_done) (void)hipFree(ctx->attn_done);
         (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return (int32_t)e;
@@ -69,6 +73,7 @@ int32_t galois_hip_destroy(galois_hip_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->attn_done) (void)hipFree(ctx->attn_done);
     hipError_t e = hipStreamDestroy(ctx->stream);
     delete ctx;
     return (int32_t)e;

@@ -212,9 +212,9 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
             G_TRY(galois_matmul(l.wk, a_, k_));
             G_TRY(galois_matmul(l.wv, a_, v_)); ops += 3;
         }
-        if (fused >= 3) {  // the eight attention ops as two launches, then the grouped tail of the layer
+        if (fused >= 3) {  // the eight attention ops as one launch, then the grouped tail of the layer
             G_TRY(galois_attn_decode(rope, q_, k_, v_, l.k_cache, l.v_cache, pos_, ao_, H, n_past, *(const float *)scale_.data()));
-            ops += L > 128 ? 2 : 1;
+            ops++;
             MatvecItem mo = item(l.wo, ao_, x1_);
             mo.residual = &x_;
             G_TRY(galois_matvec_group({mo})); ops++;

@@ -105,6 +105,34 @@ def test_attn_decode_invariants(dev):
     assert emax < TOL and el2 < TOL
 
 
+def test_attn_decode_repeated_calls_merge_fresh_partials(dev):
+    """The splits of a head are merged by whichever workgroup finishes last, reading the other workgroups' records
+    from a block that every call reuses: back-to-back calls with different values must each merge their own."""
+    H, D, L = 32, 128, 1500          # 12 splits per head
+    rng = np.random.default_rng(21)
+    fs, ts, scale = 1.0, float(np.float32(10000.0) ** np.float32(-2.0 / D)), float(1.0 / np.sqrt(D))
+    kc = rng.standard_normal((L, H * D)).astype(np.float32)
+    vc0 = rng.standard_normal((L, H * D)).astype(np.float32)
+    q, k = (rng.standard_normal(H * D).astype(np.float32) for _ in range(2))
+    pos = dev.upload(np.array([L - 1], np.int32))
+    qb, kb, kcb = dev.upload(q), dev.upload(k), dev.upload(kc)
+    outs, vbufs, vhost = [], [], []
+    for i in range(12):            # values scaled differently per call, no synchronisation in between
+        vc = (vc0 * np.float32(1.0 + i)).astype(np.float32)
+        vhost.append(vc)
+        vbufs.append((dev.upload(vc[L - 1].copy()), dev.upload(vc)))
+        outs.append(dev.alloc(H * D * 4))
+    for i in range(12):
+        dev.attn_decode_f32(qb, kb, vbufs[i][0], kcb, vbufs[i][1], outs[i], H, D, L - 1, pos, fs, ts, scale)
+    res = [dev.download(o, np.float32, H * D) for o in outs]
+    for i in range(1, 12):         # the output is linear in the values
+        err = np.max(np.abs(res[i] - res[0] * np.float32(1.0 + i))) / np.max(np.abs(res[i]))
+        assert err <= 1e-6, (i, err)
+    rot = (_gpu_rope(dev, q, H, D, L - 1, fs, ts), _gpu_rope(dev, k, H, D, L - 1, fs, ts))
+    ref = _ref(q, k, vhost[0][L - 1].copy(), kc.copy(), vhost[0].copy(), H, D, L - 1, fs, ts, scale, rotated=rot)
+    assert np.max(np.abs(res[0] - ref)) / np.max(np.abs(ref)) <= TOL
+
+
 def test_attn_decode_argument_errors(dev):
     buf = dev.alloc(1 << 16)
     ok = [buf, buf, buf, buf, buf, buf, 2, 64, 0, buf, 1.0, 0.9, 0.1]
