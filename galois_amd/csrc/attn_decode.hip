@@ -21,7 +21,7 @@
 namespace {
 
 constexpr int AT_THREADS = 256;
-constexpr int AT_KEYS = 128;  // keys per workgroup
+constexpr int AT_KEYS = 128;  // keys per workgroup (measured: 64 and, for an f16 cache, 256 are slower)
 
 template <int CTRL>
 __device__ __forceinline__ float at_dpp(float v) {
@@ -63,8 +63,11 @@ __device__ __forceinline__ float at_wave_sum(float v) {
 // theta = pos * freq_scale * theta_scale^i.
 struct at_rot {
     float c0, s0, c1, s1;
+    // the same sequence of roundings as rope_rows (one product, then a fused multiply-add), spelled out so that the
+    // compiler cannot contract the two kernels differently: the appended cache row equals rope_f32's output
     __device__ __forceinline__ float4 apply(float4 x) const {
-        return make_float4(x.x * c0 - x.y * s0, x.x * s0 + x.y * c0, x.z * c1 - x.w * s1, x.z * s1 + x.w * c1);
+        return make_float4(__builtin_fmaf(x.x, c0, -(x.y * s0)), __builtin_fmaf(x.x, s0, x.y * c0),
+                           __builtin_fmaf(x.z, c1, -(x.w * s1)), __builtin_fmaf(x.z, s1, x.w * c1));
     }
 };
 
@@ -122,18 +125,43 @@ __device__ __forceinline__ void at_combine(const float *rec, float *__restrict__
     }
 }
 
+// The lane's four consecutive cache elements, f32 or f16 (the reference keeps f16 caches on the GPU: cpy_f32_f16,
+// src/cuda.rs:1382-1595, then gemm_ex with F16 operands, src/cuda.rs:881-992).  Rows appended to an f16 cache are
+// rounded to nearest even, and this step's scores and outputs use the rounded row, as the op sequence would.
+typedef _Float16 at_half4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 at_load4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ at_half4 at_load4(const _Float16 *p) { return *reinterpret_cast<const at_half4 *>(p); }
+__device__ __forceinline__ float4 at_f32(float4 v) { return v; }
+__device__ __forceinline__ float4 at_f32(at_half4 h) { return make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w); }
+template <typename CT> struct at_raw { typedef float4 type; };
+template <> struct at_raw<_Float16> { typedef at_half4 type; };
+__device__ __forceinline__ float4 at_load4_rounded(float4 v) {  // v as an f16 cache returns it
+    return make_float4((float)(_Float16)v.x, (float)(_Float16)v.y, (float)(_Float16)v.z, (float)(_Float16)v.w);
+}
+__device__ __forceinline__ float4 at_store4(float *p, float4 v) {
+    *reinterpret_cast<float4 *>(p) = v;
+    return v;
+}
+__device__ __forceinline__ float4 at_store4(_Float16 *p, float4 v) {
+    const at_half4 h = {(_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w};
+    *reinterpret_cast<at_half4 *>(p) = h;
+    return make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w);
+}
+
 // Record of one (head, split) in the scratch block: m, sum, 2 unused floats, then head_dim partial outputs.
-template <int LPR>
+template <int LPR, typename CT>
 __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *__restrict__ q, const float *__restrict__ k,
-                                                                  const float *__restrict__ v, float *__restrict__ kc,
-                                                                  float *__restrict__ vc, float *__restrict__ part,
+                                                                  const float *__restrict__ v, CT *__restrict__ kc,
+                                                                  CT *__restrict__ vc, float *__restrict__ part,
                                                                   unsigned *__restrict__ done, float *__restrict__ out, int H, int L,
                                                                   const int32_t *__restrict__ pos, float freq_scale,
                                                                   float theta_scale, float scale) {
     constexpr int D = LPR * 4, RPL = 64 / LPR, WAVES = AT_THREADS / 64;
-    constexpr int KPW = AT_KEYS / WAVES;  // keys per wave
+    constexpr int KEYS = AT_KEYS;
+    constexpr int KPW = KEYS / WAVES;     // keys per wave
     constexpr int U = KPW / RPL;          // wave-loads per wave, all in flight
-    __shared__ float sc[AT_KEYS];
+    constexpr bool F16 = sizeof(CT) == 2;
+    __shared__ float sc[KEYS];
     __shared__ float4 ored[WAVES][LPR];
     __shared__ float sred[WAVES];
     __shared__ float cw[AT_MAX_SPLITS];
@@ -142,26 +170,23 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane / LPR, kl = lane % LPR;
     const int h = blockIdx.y, s = blockIdx.x, S = gridDim.x;
-    const int l0 = s * AT_KEYS, l1 = min(L, l0 + AT_KEYS), nl = l1 - l0;
+    const int l0 = s * KEYS, l1 = min(L, l0 + KEYS), nl = l1 - l0;
     const size_t E = (size_t)H * D;
     const size_t hoff = (size_t)h * D + kl * 4;
 
     const int lnew = L - 1;  // the position being appended
     const int kbase = l0 + wave * KPW + sub;
 
-    // ---- every request of the workgroup goes out first: its keys and values (the new position's come from k and
-    // v, it is not in the cache yet), then q; the rotation is computed while they are in flight
-    float4 kv[U], vv[U];
+    // ---- every request of the workgroup goes out first: its keys and values as the cache holds them (row n_past
+    // is not in the cache yet: what is read for it is replaced below by this step's k and v), then k, v and q;
+    // the rotation is computed while they are in flight
+    typename at_raw<CT>::type kv[U], vv[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int lc = min(kbase + u * RPL, l1 - 1);
-        kv[u] = *reinterpret_cast<const float4 *>(lc == lnew ? k + hoff : kc + (size_t)lc * E + hoff);
-    }
+    for (int u = 0; u < U; u++) kv[u] = at_load4(kc + (size_t)min(kbase + u * RPL, l1 - 1) * E + hoff);
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int lc = min(kbase + u * RPL, l1 - 1);
-        vv[u] = *reinterpret_cast<const float4 *>(lc == lnew ? v + hoff : vc + (size_t)lc * E + hoff);
-    }
+    for (int u = 0; u < U; u++) vv[u] = at_load4(vc + (size_t)min(kbase + u * RPL, l1 - 1) * E + hoff);
+    const float4 knew_raw = *reinterpret_cast<const float4 *>(k + hoff);
+    float4 vnew = *reinterpret_cast<const float4 *>(v + hoff);
     const float4 qraw = *reinterpret_cast<const float4 *>(q + hoff);
     // this position's rotation for the lane's pairs 2 kl and 2 kl + 1
     at_rot rot;
@@ -171,36 +196,47 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
         sincosf(p0 * powf(theta_scale, (float)(2 * kl + 1)), &rot.s1, &rot.c1);
     }
     const float4 qv = rot.apply(qraw);
+    float4 knew = rot.apply(knew_raw);
+    if (F16) {  // what an f16 cache will hold
+        // the rotation's f32 result is rounded again to f16, as a cpy of rope_custom's output is; without the
+        // barrier the compiler folds rotation and conversion into one mixed-precision fma (one rounding)
+        asm volatile("" : "+v"(knew.x), "+v"(knew.y), "+v"(knew.z), "+v"(knew.w));
+        knew = at_load4_rounded(knew);
+        vnew = at_load4_rounded(vnew);
+    }
 
     // ---- scores of the workgroup's keys
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int l = kbase + u * RPL;
-        if (min(l, l1 - 1) == lnew) {  // rotate the new key; the lanes that own it write both cache rows
-            kv[u] = rot.apply(kv[u]);
+        float4 kf = at_f32(kv[u]);
+        if (min(l, l1 - 1) == lnew) {  // the new key; the lanes that own it write both cache rows
+            kf = knew;
             if (l == lnew) {
-                *reinterpret_cast<float4 *>(kc + (size_t)lnew * E + hoff) = kv[u];
-                *reinterpret_cast<float4 *>(vc + (size_t)lnew * E + hoff) = vv[u];
+                at_store4(kc + (size_t)lnew * E + hoff, knew);
+                at_store4(vc + (size_t)lnew * E + hoff, vnew);
             }
         }
-        float acc = kv[u].x * qv.x;
-        acc = __builtin_fmaf(kv[u].y, qv.y, acc);
-        acc = __builtin_fmaf(kv[u].z, qv.z, acc);
-        acc = __builtin_fmaf(kv[u].w, qv.w, acc);
+        float acc = kf.x * qv.x;
+        acc = __builtin_fmaf(kf.y, qv.y, acc);
+        acc = __builtin_fmaf(kf.z, qv.z, acc);
+        acc = __builtin_fmaf(kf.w, qv.w, acc);
         acc = at_group_sum<LPR>(acc);
         if (kl == 0) sc[wave * KPW + u * RPL + sub] = acc * scale;
     }
     __syncthreads();
 
     // ---- softmax numerators relative to the workgroup's own maximum
-    float m;
-    {
-        const float ninf = -__builtin_inff();
-        const float a = lane < nl ? sc[lane] : ninf, b = lane + 64 < nl ? sc[lane + 64] : ninf;
-        m = at_wave_max(fmaxf(a, b));
-    }
+    float m = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < KEYS; i += 64) m = fmaxf(m, lane + i < nl ? sc[lane + i] : -__builtin_inff());
+    m = at_wave_max(m);
     __syncthreads();  // every wave has read the scores
-    if (threadIdx.x < AT_KEYS) sc[threadIdx.x] = (int)threadIdx.x < nl ? expf(sc[threadIdx.x] - m) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < KEYS; i += AT_THREADS) {
+        const int j = (int)threadIdx.x + i;
+        sc[j] = j < nl ? expf(sc[j] - m) : 0.0f;
+    }
     __syncthreads();
 
     // ---- partial output: sum of p * v over the workgroup's keys (p is 0 for keys past the end)
@@ -208,10 +244,11 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const float p = sc[wave * KPW + u * RPL + sub];
-        acc.x = __builtin_fmaf(vv[u].x, p, acc.x);
-        acc.y = __builtin_fmaf(vv[u].y, p, acc.y);
-        acc.z = __builtin_fmaf(vv[u].z, p, acc.z);
-        acc.w = __builtin_fmaf(vv[u].w, p, acc.w);
+        const float4 vf = min(kbase + u * RPL, l1 - 1) == lnew ? vnew : at_f32(vv[u]);
+        acc.x = __builtin_fmaf(vf.x, p, acc.x);
+        acc.y = __builtin_fmaf(vf.y, p, acc.y);
+        acc.z = __builtin_fmaf(vf.z, p, acc.z);
+        acc.w = __builtin_fmaf(vf.w, p, acc.w);
     }
     // the RPL keys of a wave-load sit LPR lanes apart
 #pragma unroll
@@ -222,7 +259,10 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
         acc.w += __shfl_xor(acc.w, off, 64);
     }
     if (lane < LPR) ored[wave][lane] = acc;
-    const float psum = at_wave_sum((lane < nl ? sc[lane] : 0.0f) + (lane + 64 < nl ? sc[lane + 64] : 0.0f));
+    float psum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < KEYS; i += 64) psum += lane + i < nl ? sc[lane + i] : 0.0f;
+    psum = at_wave_sum(psum);
     if (lane == 0) sred[wave] = psum;  // every wave holds the same total; wave 0's is used
     __syncthreads();
     if (wave == 0 && lane < LPR) {
@@ -261,34 +301,51 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
     at_combine(part + (size_t)h * S * (D + 4), out + (size_t)h * D, D, S, cw, cred);
 }
 
-}  // namespace
 
-extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
-                                              float *k_cache, float *v_cache, float *out, int32_t n_head,
-                                              int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
-                                              float theta_scale, float scale) {
+template <typename CT>
+int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, CT *k_cache, CT *v_cache,
+                           float *out, int32_t n_head, int32_t head_dim, int32_t n_past, const int32_t *pos,
+                           float freq_scale, float theta_scale, float scale, const char *what) {
     GH_REQUIRE_CTX(ctx);
-    GH_REQUIRE(ctx, q && k && v && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, "attn_decode_f32");
+    GH_REQUIRE(ctx, q && k && v && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, what);
     GH_REQUIRE(ctx, n_head > 0 && n_head <= 65535 && n_past >= 0 && n_past < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
-               "attn_decode_f32: n_head in 1..65535, n_past >= 0");
-    GH_REQUIRE(ctx, head_dim == 64 || head_dim == 128, GALOIS_HIP_E_UNSUPPORTED, "attn_decode_f32: head_dim 64 or 128");
+               "attn_decode: n_head in 1..65535, n_past >= 0");
+    GH_REQUIRE(ctx, head_dim == 64 || head_dim == 128, GALOIS_HIP_E_UNSUPPORTED, "attn_decode: head_dim 64 or 128");
     GH_REQUIRE(ctx, gh_aligned(q, 16) && gh_aligned(k, 16) && gh_aligned(v, 16) && gh_aligned(k_cache, 16) &&
                         gh_aligned(v_cache, 16) && gh_aligned(out, 16) && gh_aligned(pos, 4),
-               GALOIS_HIP_E_ALIGN, "attn_decode_f32: 16-byte aligned vectors and caches");
+               GALOIS_HIP_E_ALIGN, "attn_decode: 16-byte aligned vectors and caches");
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
     GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && (int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr && ctx->attn_done != nullptr),
-               GALOIS_HIP_E_UNSUPPORTED, "attn_decode_f32: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
+               GALOIS_HIP_E_UNSUPPORTED, "attn_decode: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
                                          "results must fit the context's 4 MB scratch block");
     GH_BIND(ctx);
     float *part = (float *)ctx->scratch;
     unsigned *done = ctx->attn_done;  // one counter per head, zero between calls
     const dim3 grid((unsigned)S, (unsigned)n_head), block(AT_THREADS);
     if (head_dim == 128)
-        hipLaunchKernelGGL(attn_decode_partial<32>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done, out,
-                           n_head, L, pos, freq_scale, theta_scale, scale);
+        hipLaunchKernelGGL((attn_decode_partial<32, CT>), grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done,
+                           out, n_head, L, pos, freq_scale, theta_scale, scale);
     else
-        hipLaunchKernelGGL(attn_decode_partial<16>, grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done, out,
-                           n_head, L, pos, freq_scale, theta_scale, scale);
-    GH_LAUNCH_CHECK(ctx, "attn_decode_f32 launch");
+        hipLaunchKernelGGL((attn_decode_partial<16, CT>), grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done,
+                           out, n_head, L, pos, freq_scale, theta_scale, scale);
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
+}  // namespace
+
+extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
+                                              float *k_cache, float *v_cache, float *out, int32_t n_head,
+                                              int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
+                                              float theta_scale, float scale) {
+    return attn_decode_launch<float>(ctx, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale,
+                                     theta_scale, scale, "attn_decode_f32");
+}
+
+extern "C" int32_t galois_hip_attn_decode_f16kv(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
+                                                void *k_cache, void *v_cache, float *out, int32_t n_head,
+                                                int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
+                                                float theta_scale, float scale) {
+    return attn_decode_launch<_Float16>(ctx, q, k, v, (_Float16 *)k_cache, (_Float16 *)v_cache, out, n_head, head_dim,
+                                        n_past, pos, freq_scale, theta_scale, scale, "attn_decode_f16kv");
 }

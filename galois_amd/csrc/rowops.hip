@@ -149,12 +149,12 @@ __global__ __launch_bounds__(kRopeThreads) void rope_rows(const float *__restric
 #pragma unroll
             for (int u = 0; u < 4; u++)
                 reinterpret_cast<float2 *>(y + (size_t)(r + u * (kRopeThreads / 64)) * ncols)[pi] =
-                    make_float2(v[u].x * cs - v[u].y * sn, v[u].x * sn + v[u].y * cs);
+                    make_float2(__builtin_fmaf(v[u].x, cs, -(v[u].y * sn)), __builtin_fmaf(v[u].x, sn, v[u].y * cs));
         }
         for (; r < row_hi; r += kRopeThreads / 64) {
             const float2 v = reinterpret_cast<const float2 *>(x + (size_t)r * ncols)[pi];
             reinterpret_cast<float2 *>(y + (size_t)r * ncols)[pi] =
-                make_float2(v.x * cs - v.y * sn, v.x * sn + v.y * cs);
+                make_float2(__builtin_fmaf(v.x, cs, -(v.y * sn)), __builtin_fmaf(v.x, sn, v.y * cs));
         }
     }
 }

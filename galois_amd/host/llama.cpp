@@ -77,7 +77,10 @@ GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Te
         if (!dev) dev = t->device().gpu;
         if (t->device().gpu != dev) return err(GError::Unimplemented, "galois_attn_decode: one device");
         if (!t->dim().ggml_is_contiguous(t->dtype())) return err(GError::Unimplemented, "galois_attn_decode: contiguous tensors only");
-        if (t->dtype() != (t == &pos ? GGmlType::I32 : GGmlType::F32)) return err(GError::Unimplemented, "galois_attn_decode: F32 tensors, I32 pos");
+        const bool cache = t == (const Tensor *)&k_cache || t == (const Tensor *)&v_cache;
+        const GGmlType want = t == &pos ? GGmlType::I32 : (cache ? k_cache.dtype() : GGmlType::F32);
+        if (t->dtype() != want || (cache && want != GGmlType::F32 && want != GGmlType::F16))
+            return err(GError::Unimplemented, "galois_attn_decode: F32 vectors, I32 pos, both caches F32 or both F16");
     }
     if (op.mode != 0) return err(GError::Unimplemented, "galois_attn_decode: rope mode 0 only (src/cuda.rs:1336-1340)");
     const size_t E = q.dim().elem_count();
@@ -86,6 +89,11 @@ GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Te
         n_past < 0 || (size_t)n_past >= k_cache.dim().shape[1] || (size_t)n_past >= v_cache.dim().shape[1])
         return err(GError::ShapeError, "galois_attn_decode: q, k, v, out of n_head * n_dims elements, caches [that, n_ctx], n_past < n_ctx");
     const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);  // as galois_rope_custom derives it (src/cuda.rs:1327)
+    if (k_cache.dtype() == GGmlType::F16)
+        return dev->check(galois_hip_attn_decode_f16kv(dev->ctx(), (const float *)q.data(), (const float *)k.data(),
+                                                       (const float *)v.data(), k_cache.data(), v_cache.data(), (float *)out.data(),
+                                                       (int32_t)n_head, (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(),
+                                                       op.freq_scale, theta_scale, scale));
     return dev->check(galois_hip_attn_decode_f32(dev->ctx(), (const float *)q.data(), (const float *)k.data(), (const float *)v.data(),
                                                  (float *)k_cache.data(), (float *)v_cache.data(), (float *)out.data(), (int32_t)n_head,
                                                  (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
@@ -120,8 +128,8 @@ GResult LlamaDecoder::create(const LlamaHParams &hp, const Device &dev, std::uni
         G_TRY(mk(&l.w_gate, Q, dev, E, F));
         G_TRY(mk(&l.w_up, Q, dev, E, F));
         G_TRY(mk(&l.w_down, Q, dev, F, E));
-        G_TRY(mk(&l.k_cache, F32, dev, E, C));
-        G_TRY(mk(&l.v_cache, F32, dev, E, C));
+        G_TRY(mk(&l.k_cache, hp.kv_f16 ? GGmlType::F16 : F32, dev, E, C));
+        G_TRY(mk(&l.v_cache, hp.kv_f16 ? GGmlType::F16 : F32, dev, E, C));
     }
     G_TRY(mk(&m->tok_id_, GGmlType::I32, dev, 1));
     G_TRY(mk(&m->pos_, GGmlType::I32, dev, 1));
@@ -172,6 +180,8 @@ GResult LlamaDecoder::set_inputs(int32_t token, int32_t n_past) {
 // The op sequence of one token.  Shapes in ggml order [ne0, ne1, ne2]; L = n_past + 1 keys are visible,
 // so the softmax needs no mask.
 GResult LlamaDecoder::step(int32_t n_past, int fused) {
+    if (hp_.kv_f16 && fused < 3)
+        return err(GError::Unimplemented, "LlamaDecoder: an f16 KV cache runs with the fused attention only (fused = 3)");
     const size_t E = hp_.n_embd, H = hp_.n_head, D = E / H, L = (size_t)n_past + 1, C = hp_.n_ctx;
     RopeCustomOption rope;
     rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;

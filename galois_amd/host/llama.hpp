@@ -17,6 +17,7 @@ namespace galois {
 struct LlamaHParams {
     size_t n_vocab = 32000, n_embd = 4096, n_head = 32, n_layer = 32, n_ff = 11008, n_ctx = 2048;
     float rms_eps = 1e-6f, freq_base = 10000.0f, freq_scale = 1.0f;
+    bool kv_f16 = false;  // KV cache in f16 (as the reference keeps it on the GPU); needs the fused attention (fused = 3)
 };
 
 class LlamaDecoder {
@@ -36,7 +37,8 @@ class LlamaDecoder {
     // rms_norm*weight and silu*up kernels instead of two ops each.
     // fused = 2 additionally sends the Q4_0 matrix-vector products out in grouped launches (q | k | v together,
     // gate | up as a SwiGLU pair) with the norms, silu * up and the residual adds riding along: 12 launches per layer;
-    // fused = 3 also replaces the eight attention ops of a layer by galois_attn_decode: 5 launches per layer.
+    // fused = 3 also replaces the eight attention ops of a layer by galois_attn_decode: 5 launches per layer
+    // (the only plan that runs with an f16 KV cache).
     GResult decode(int32_t token, int32_t n_past, int fused);
     // Records the same step as a graph / replays the recorded step.
     GResult capture(int32_t token, int32_t n_past, int fused);
@@ -79,7 +81,7 @@ struct MatvecItem {
 GResult galois_matvec_group(const std::vector<MatvecItem> &items);
 
 // Attention of one decode step in one launch (galois_hip_attn_decode_f32): rope_custom of q and k at position
-// pos[0] = n_past, append of k and v to row n_past of the caches ([n_embd, n_ctx] f32 each), scores = K^T q scaled
+// pos[0] = n_past, append of k and v to row n_past of the caches ([n_embd, n_ctx], both f32 or both f16), scores = K^T q scaled
 // by `scale`, soft_max over the n_past + 1 keys and out = V p, for n_head heads of q.dim / n_head elements.
 GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                            Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale);

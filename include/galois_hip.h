@@ -224,6 +224,14 @@ int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const fl
                                    float *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
                                    const int32_t *pos, float freq_scale, float theta_scale, float scale);
 
+/* The same with f16 caches, the form the reference keeps them in on the GPU (cpy_f32_f16 into the cache,
+ * src/cuda.rs:1382-1595, then gemm_ex on F16 operands, src/cuda.rs:881-992): k_cache, v_cache are
+ * [n_ctx][n_head * head_dim] f16; row n_past receives rope(k) and v rounded to nearest even, and this step's scores
+ * and output use the rounded row, as a cpy followed by the matmuls would.  Half the cache bytes per step. */
+int32_t galois_hip_attn_decode_f16kv(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, void *k_cache,
+                                     void *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
+                                     const int32_t *pos, float freq_scale, float theta_scale, float scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,35 @@ def test_attn_decode_matches_the_op_sequence(dev, H, D, n_ctx, n_past):
     assert emax < TOL_ROPE
 
 
+@pytest.mark.parametrize("H,D,n_ctx,n_past", [(32, 128, 2048, 2047), (32, 128, 300, 128), (2, 64, 64, 37), (5, 64, 1000, 0)])
+def test_attn_decode_with_f16_caches(dev, H, D, n_ctx, n_past):
+    """f16 caches: the appended rows are rope(k) and v rounded to nearest even, and the step computes with the
+    rounded rows, like cpy_f32_f16 into the cache followed by the matmuls on its f16 contents."""
+    rng = np.random.default_rng(H * 77 + D + n_past)
+    E = H * D
+    q, k, v = (rng.standard_normal(E).astype(np.float32) for _ in range(3))
+    kc16 = rng.standard_normal((n_ctx, E)).astype(np.float16)
+    vc16 = rng.standard_normal((n_ctx, E)).astype(np.float16)
+    fs, ts, scale = 1.0, float(np.float32(10000.0) ** np.float32(-2.0 / D)), 1.0 / np.sqrt(D)
+    bufs = [dev.upload(a) for a in (q, k, v, kc16, vc16)]
+    out, pos = dev.alloc(E * 4), dev.upload(np.array([n_past], np.int32))
+    dev.attn_decode_f16kv(bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], out, H, D, n_past, pos, fs, ts, scale)
+    got = dev.download(out, np.float32, E)
+    kc_g, vc_g = dev.download(bufs[3], np.float16, kc16.shape), dev.download(bufs[4], np.float16, vc16.shape)
+    qr, kr = _gpu_rope(dev, q, H, D, n_past, fs, ts), _gpu_rope(dev, k, H, D, n_past, fs, ts)
+    rows = np.arange(n_ctx) != n_past
+    assert np.array_equal(kc_g[rows], kc16[rows]) and np.array_equal(vc_g[rows], vc16[rows])
+    assert np.array_equal(kc_g[n_past], kr.astype(np.float16)) and np.array_equal(vc_g[n_past], v.astype(np.float16))
+    # the op sequence on the oracle over the f16 contents: rotated k and v already rounded as the cache holds them
+    kc32, vc32 = kc16.astype(np.float32), vc16.astype(np.float32)
+    ref = _ref(q, kr.astype(np.float16).astype(np.float32), v.astype(np.float16).astype(np.float32), kc32, vc32, H, D, n_past,
+               fs, ts, scale, rotated=(qr, kr.astype(np.float16).astype(np.float32)))
+    emax, el2 = npref.rel_err(got, ref)
+    assert emax < TOL and el2 < TOL, (emax, el2)
+    for b in bufs + [out, pos]:
+        dev.free(b)
+
+
 def test_attn_decode_invariants(dev):
     """One key: the output is that key's value row whatever q is.  Equal keys: the mean of the values."""
     H, D, n_ctx = 4, 128, 512

@@ -39,8 +39,9 @@ def _load(dec, w, kc=None, vc=None):
             dec.tensor("v_cache", i).write(vc[i])
 
 
-def _ref_step(w, hp, kc, vc, token, n_past):
-    """One token through the oracle's ops; kc / vc [n_layer][n_ctx][n_embd] are updated in place."""
+def _ref_step(w, hp, kc, vc, token, n_past, round_kv=False):
+    """One token through the oracle's ops; kc / vc [n_layer][n_ctx][n_embd] are updated in place.
+    round_kv: the appended rows are rounded to f16 (an f16 cache) before the attention reads them."""
     e, h = hp["n_embd"], hp["n_head"]
     d, L, eps = e // h, n_past + 1, hp["rms_eps"]
     theta_scale = np.float32(hp["freq_base"]) ** np.float32(-2.0 / d)
@@ -52,6 +53,9 @@ def _ref_step(w, hp, kc, vc, token, n_past):
         qr = oracle.rope(q.reshape(h, d), pos, 1.0, h, float(theta_scale))
         kr = oracle.rope(k.reshape(h, d), pos, 1.0, h, float(theta_scale))
         kc[i][n_past], vc[i][n_past] = kr.reshape(-1), v
+        if round_kv:
+            kc[i][n_past] = kc[i][n_past].astype(np.float16).astype(np.float32)
+            vc[i][n_past] = vc[i][n_past].astype(np.float16).astype(np.float32)
         kview = np.lib.stride_tricks.as_strided(kc[i], (h, L, d), (d * 4, e * 4, 4))
         s = oracle.mul_mat_f32(kview, qr.reshape(h, 1, d))                       # [h, 1, L]
         p = oracle.soft_max(oracle.scale(s, float(np.float32(1.0) / np.sqrt(np.float32(d)))).reshape(h, L))
@@ -119,6 +123,30 @@ def test_decode_from_an_empty_cache_over_several_tokens(gdev):
         ref = _ref_step(w, hp, kc, vc, tok, n_past)
         dec.decode(tok, n_past, (0, 3, 2, 1, 3)[n_past])   # every launch plan in turn, on one cache
         _check(dec.logits(), ref, 1e-4)
+    dec.close()
+
+
+def test_decode_with_an_f16_kv_cache(gdev):
+    """KV cache in f16 (fused attention only): logits against the oracle's step run on caches rounded to f16 after
+    every append, over several tokens on one cache."""
+    rng = np.random.default_rng(53)
+    hp = SMALL
+    w = _make_weights(rng, hp)
+    dec = g.LlamaDecoder(gdev, kv_f16=True, **hp)
+    _load(dec, w)
+    kc = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float32)
+    vc = np.zeros_like(kc)
+    for n_past, tok in enumerate([5, 300, 41, 41]):
+        # the oracle's step appends f32 rows; this step's own attention must already see them rounded
+        ref = _ref_step(w, hp, kc, vc, tok, n_past, round_kv=True)
+        dec.decode(tok, n_past, 3)
+        _check(dec.logits(), ref, 2e-4)
+    kg = dec.tensor("k_cache", 1).to_cpu_tensor()
+    assert kg.dtype == np.float16 and np.array_equal(kg[4:], np.zeros_like(kg[4:])) and np.any(kg[3] != 0)
+    _check(kg[:4].astype(np.float32), kc[1][:4], 1e-3)
+    with pytest.raises(g.GError) as e:
+        dec.decode(1, 4, 2)
+    assert e.value.kind == "Unimplemented"
     dec.close()
 
 
