@@ -153,6 +153,23 @@ def test_group_swiglu_pair_and_residual(dev, k, n):
     _check(a, oracle.silu(g).astype(np.float64) * u, "swiglu, oracle ops")
 
 
+def test_group_of_six_with_norm_pairs_and_residuals(dev):
+    """More than four products per launch take the kernel build that selects among eight argument sets."""
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal(256).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(256)).astype(np.float32)
+    items = []
+    for i, n in enumerate([33, 1, 700, 64, 129, 16]):
+        it = {"vx": _wx(100 + i, 256, n), "y": x, "norm_weight": g, "norm_eps": 1e-5}
+        if i % 2 == 0:
+            it["vx_up"] = _wx(200 + i, 256, n)
+        if i % 3 == 0:
+            it["residual"] = rng.standard_normal(n).astype(np.float32)
+        items.append(it)
+    for i, (it, got) in enumerate(zip(items, _run_group(dev, items))):
+        _check(got, _ref_item(it), i)
+
+
 def test_group_special_values(dev):
     k, n = 4096, 40
     wq = _wx(99, k, n)
