@@ -133,7 +133,8 @@ __global__ __launch_bounds__(256) void gemm_q4_0_mfma_v1(const uint8_t *__restri
 //     in registers, and 4 producers that fetch the weights as whole 144-byte row pieces (4 stages at
 //     a time), park them raw in LDS, and each stage dequantise one slot per row into an fp16 B tile
 //     that all four consumers read.  Each SIMD hosts one wave of each kind.
-//     (-DGEMM_TILE_N=176 builds the earlier 128 x 176 tile with the consumers as 2 x 2.)
+//     For narrow matrices the tile is 256 x 48 (3 MFMA tiles per wave in N): N = 4096 at M = 512 is 86
+//     workgroups of 96 columns but 172 of 48.
 //   - The fp16 B tile is triple-buffered, one barrier per stage: while the consumers multiply the
 //     second k-half of stage s they already hold the first half of stage s+1, and the producers
 //     write stage s+2.  LDS carries only B.
@@ -142,15 +143,21 @@ __global__ __launch_bounds__(256) void gemm_q4_0_mfma_v1(const uint8_t *__restri
 //     six matrix instructions instead of in bursts.
 //   - blockIdx is mapped so that an XCD (blockIdx % 8) owns one 256-row panel of X and a
 //     contiguous range of weight tiles: X stays in that XCD's L2, W streams once per panel.
-#ifndef GEMM_TILE_N
-#define GEMM_TILE_N 96
-#endif
-constexpr int GN = GEMM_TILE_N;           // 96: four consumer waves stacked in M (tile 256 x 96); 176: 2 x 2 (tile 128 x 176)
-constexpr int GM = GN == 96 ? 256 : 128;
-constexpr int GTASKS = (GN * 4 + 255) / 256;  // dequantisation tasks per producer thread and stage
+// The N extent of the tile is a template parameter: 96 columns (6 MFMA tiles per consumer wave) for wide
+// matrices, 48 (3 per wave) when 96 would leave most CUs without a workgroup (N = 4096 at M = 512: 86 tiles).
+constexpr int GM = 256;
 constexpr int GBSTRIDE = 80;                  // halfs per B row in LDS: 160-byte rows
-constexpr int GB_HALFS = GN * GBSTRIDE;       // 14,080 halfs (28,160 B) per stage buffer
 constexpr int GNBUF = 3;
+constexpr int GRAW_STRIDE = 144;              // raw bytes per tile row per super-stage (4 slots)
+template <int GN>
+struct gemm_cfg {
+    static constexpr int TASKS = (GN * 4 + 255) / 256;  // dequantisation tasks per producer thread and stage
+    static constexpr int B_HALFS = GN * GBSTRIDE;       // halfs per stage buffer (15,360 B for 96 columns)
+    static constexpr int RAW_BYTES = GN * GRAW_STRIDE;  // bytes per raw buffer (13,824 B for 96 columns)
+    static constexpr int RAW_CHUNKS = GN * 9;           // 16-byte chunks per raw buffer
+    static constexpr int RAW_PER_THREAD = (RAW_CHUNKS + 255) / 256;
+    static constexpr size_t LDS_BYTES = (size_t)GNBUF * B_HALFS * sizeof(_Float16) + 2 * (size_t)RAW_BYTES + 16;
+};
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 // X -> fp16 in the order the MFMA A operand is fetched: tiles of 16 rows x 32 k (1 KB), tile (m16, kb)
@@ -199,11 +206,6 @@ __device__ __forceinline__ void deq_dword(uint32_t v, half2_t d2, uint32_t lo[2]
 // The weights are fetched four stages at a time as the 144 contiguous bytes (8 blocks) each
 // tile row contributes: nine consecutive lanes read one row piece with 16-byte loads, so every
 // request is made of whole lines.  The pieces are parked as raw bytes in LDS.
-constexpr int GRAW_STRIDE = 144;                 // raw bytes per tile row per super-stage (4 slots)
-constexpr int GRAW_BYTES = GN * GRAW_STRIDE;     // 25,344 B per raw buffer
-constexpr int GRAW_CHUNKS = GN * 9;              // 16-byte chunks per raw buffer
-constexpr int GRAW_PER_THREAD = (GRAW_CHUNKS + 255) / 256;
-constexpr size_t GEMM_LDS_BYTES = (size_t)GNBUF * GB_HALFS * sizeof(_Float16) + 2 * (size_t)GRAW_BYTES + 16;
 
 // Global loads whose use is a loop iteration (or four) away are issued through inline assembly and
 // waited for by hand: loads retire in order, so "at most n younger loads outstanding" is the exact
@@ -215,25 +217,28 @@ __device__ __forceinline__ void gload16(u32x4_t &dst, const void *ptr) {
 }
 #define GEMM_VMWAIT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
 
+template <int GN>
 struct gemm_raw_regs {
-    u32x4_t c[GRAW_PER_THREAD];
+    u32x4_t c[gemm_cfg<GN>::RAW_PER_THREAD];
 };
 
+template <int GN>
 __device__ __forceinline__ void gemm_load_raw(const uint8_t *W, size_t wrow_bytes, int N, int n0, int p, int super,
-                                              gemm_raw_regs &r) {
+                                              gemm_raw_regs<GN> &r) {
 #pragma unroll
-    for (int i = 0; i < GRAW_PER_THREAD; i++) {
-        const int q = min(p + 256 * i, GRAW_CHUNKS - 1);
+    for (int i = 0; i < gemm_cfg<GN>::RAW_PER_THREAD; i++) {
+        const int q = min(p + 256 * i, gemm_cfg<GN>::RAW_CHUNKS - 1);
         const int row = q / 9, c = q - row * 9;
         gload16(r.c[i], W + (size_t)min(n0 + row, N - 1) * wrow_bytes + (size_t)super * GRAW_STRIDE + c * 16);
     }
 }
 
-__device__ __forceinline__ void gemm_store_raw(uint8_t *raw, int p, const gemm_raw_regs &r) {
+template <int GN>
+__device__ __forceinline__ void gemm_store_raw(uint8_t *raw, int p, const gemm_raw_regs<GN> &r) {
 #pragma unroll
-    for (int i = 0; i < GRAW_PER_THREAD; i++) {
+    for (int i = 0; i < gemm_cfg<GN>::RAW_PER_THREAD; i++) {
         const int q = p + 256 * i;
-        if (q < GRAW_CHUNKS) *reinterpret_cast<u32x4_t *>(raw + q * 16) = r.c[i];
+        if (q < gemm_cfg<GN>::RAW_CHUNKS) *reinterpret_cast<u32x4_t *>(raw + q * 16) = r.c[i];
     }
 }
 
@@ -244,14 +249,15 @@ __device__ __forceinline__ void gemm_store_raw(uint8_t *raw, int p, const gemm_r
 // eight consecutive lanes fall into 32 different banks.
 // The raw bytes of a stage are read from LDS one stage ahead (gemm_stage_read) and turned into fp16
 // after the barrier (gemm_stage_write), so that the read latency is not on the path between two barriers.
+template <int GN>
 struct gemm_stage_regs {
-    uint32_t dbits[GTASKS], w0[GTASKS], w1[GTASKS], w2[GTASKS];
+    uint32_t dbits[gemm_cfg<GN>::TASKS], w0[gemm_cfg<GN>::TASKS], w1[gemm_cfg<GN>::TASKS], w2[gemm_cfg<GN>::TASKS];
 };
 
-template <int J>
-__device__ __forceinline__ void gemm_stage_read(gemm_stage_regs &r, const uint8_t *raw, int p) {
+template <int J, int GN>
+__device__ __forceinline__ void gemm_stage_read(gemm_stage_regs<GN> &r, const uint8_t *raw, int p) {
 #pragma unroll
-    for (int it = 0; it < GTASKS; it++) {
+    for (int it = 0; it < gemm_cfg<GN>::TASKS; it++) {
         const int q = p + 256 * it;
         if ((it + 1) * 256 <= GN * 4 || q < GN * 4) {
             const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
@@ -264,9 +270,10 @@ __device__ __forceinline__ void gemm_stage_read(gemm_stage_regs &r, const uint8_
     }
 }
 
-__device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs &r, _Float16 *Bs, int p) {
+template <int GN>
+__device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs<GN> &r, _Float16 *Bs, int p) {
 #pragma unroll
-    for (int it = 0; it < GTASKS; it++) {
+    for (int it = 0; it < gemm_cfg<GN>::TASKS; it++) {
         const int q = p + 256 * it;
         if ((it + 1) * 256 <= GN * 4 || q < GN * 4) {
             const int row = q >> 2, b = (q >> 1) & 1, jp = q & 1;
@@ -287,7 +294,9 @@ __device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs &r, _Floa
 
 // Barrier protocol (both kinds of wave meet every one): R after the first raw piece is parked,
 // then barrier t after stage t is written, for t = 0 .. nslots-1.  Stage t goes to buffer t % 3.
+template <int GN>
 __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__restrict__ W, int K, int N, int n0) {
+    constexpr int GB_HALFS = gemm_cfg<GN>::B_HALFS, GRAW_BYTES = gemm_cfg<GN>::RAW_BYTES;
     const int p = threadIdx.x - 256;
     const int nslots = K / 64;            // stages; a multiple of 4 (K % 256 == 0)
     const int nsuper = nslots / 4;
@@ -300,13 +309,13 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
     for (int t = 0; t < nslots; t++) __syncthreads();
     return;
 #endif
-    gemm_raw_regs rr;
+    gemm_raw_regs<GN> rr;
     gemm_load_raw(W, wrow_bytes, N, n0, p, 0, rr);
     GEMM_VMWAIT(0);
     gemm_store_raw(raw0, p, rr);
     gemm_load_raw(W, wrow_bytes, N, n0, p, min(1, nsuper - 1), rr);
     __syncthreads();  // R
-    gemm_stage_regs s0, s1;
+    gemm_stage_regs<GN> s0, s1;
     gemm_stage_read<0>(s0, raw0, p);
     for (int sup = 0; sup < nsuper; sup++) {
         const uint8_t *raw = (sup & 1) ? raw1 : raw0;
@@ -335,7 +344,7 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
     // be overwritten when it lands.  Drain, then name every register so all stay allocated until here.
     GEMM_VMWAIT(0);
 #pragma unroll
-    for (int i = 0; i < GRAW_PER_THREAD; i++) asm volatile("" ::"v"(rr.c[i]));
+    for (int i = 0; i < gemm_cfg<GN>::RAW_PER_THREAD; i++) asm volatile("" ::"v"(rr.c[i]));
 }
 
 // ---- consumer side -----------------------------------------------------------------------
@@ -386,10 +395,11 @@ __device__ __forceinline__ void gemm_load_a1(u32x4_t &dst, const _Float16 *xs, u
 #else
 #define GEMM_XKEEP
 #endif
-template <int NF>
+template <int NF, int GN>
 __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float16 *__restrict__ Xh,
                                               float *__restrict__ Y, int K, int N, int M, int m0, int n0, int wm,
                                               int ncol0) {
+    constexpr int GB_HALFS = gemm_cfg<GN>::B_HALFS;
     const int lane = threadIdx.x & 63;
     const int nslots = K / 64;
     float4_t acc[4][NF];
@@ -493,6 +503,7 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
         }
 }
 
+template <int GN>
 __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict__ W, const _Float16 *__restrict__ Xh,
                                                       float *__restrict__ Y, int K, int N, int M, int n_tiles,
                                                       int m_tiles) {
@@ -506,13 +517,26 @@ __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict_
     const int m0 = mt * GM, n0 = nt * GN;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (wave >= 4)
-        gemm_producer(smem, W, K, N, n0);
-    else if (GN == 96)  // four consumer waves stacked in M, each 64 rows x 96 columns
-        gemm_consumer<6>(smem, Xh, Y, K, N, M, m0, n0, wave, 0);
-    else if ((wave & 1) == 0)  // 2 (M) x 2 (N): the left column owns 6 column tiles (96 wide), the right one 5 (80)
-        gemm_consumer<6>(smem, Xh, Y, K, N, M, m0, n0, wave >> 1, 0);
-    else
-        gemm_consumer<5>(smem, Xh, Y, K, N, M, m0, n0, wave >> 1, 96);
+        gemm_producer<GN>(smem, W, K, N, n0);
+    else  // four consumer waves stacked in M, each 64 rows x GN columns
+        gemm_consumer<GN / 16, GN>(smem, Xh, Y, K, N, M, m0, n0, wave, 0);
+}
+
+// Launch of one tile width; the attribute that lifts the dynamic LDS limit is set once per instantiation.
+template <int GN>
+int32_t gemm_launch(galois_hip_ctx *ctx, const uint8_t *W, const _Float16 *Xh, float *Y, int K, int N, int M) {
+    const int n_tiles = (N + GN - 1) / GN, m_tiles = (M + GM - 1) / GM;
+    const int total = n_tiles * m_tiles;
+    const int grid = ((total + 7) / 8) * 8;
+    const size_t lds = gemm_cfg<GN>::LDS_BYTES;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_q4_0_mfma<GN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(gemm_q4_0_mfma<GN>, dim3(grid), dim3(512), lds, ctx->stream, W, Xh, Y, K, N, M, n_tiles, m_tiles);
+    return GALOIS_HIP_OK;
 }
 
 }  // namespace
@@ -546,19 +570,18 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
         const int64_t nchunks = m_pad * K / 8;
         hipLaunchKernelGGL(f32_to_f16_tiles, dim3((unsigned)((nchunks + 255) / 256)), dim3(256), 0, ctx->stream, X, Xh, M,
                            K, nchunks);
-        const int n_tiles = (N + GN - 1) / GN, m_tiles = (M + GM - 1) / GM;
-        const int total = n_tiles * m_tiles;
-        const int grid = ((total + 7) / 8) * 8;
-        const size_t lds = GEMM_LDS_BYTES;
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void *)gemm_q4_0_mfma, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)lds);
-            if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
-            attr_set = true;
-        }
-        hipLaunchKernelGGL(gemm_q4_0_mfma, dim3(grid), dim3(512), lds, ctx->stream, (const uint8_t *)W, Xh, Y, K, N, M,
-                           n_tiles, m_tiles);
+        // Tile width by how many workgroups it gives the device.  Cost model: rounds of workgroups over the CUs
+        // times the relative cost of a k-stage (a 48-column stage has half the matrix instructions and half
+        // the dequantisation of a 96-column one but the same barriers and A requests: ~0.65).
+        const int64_t m_tiles = (M + GM - 1) / GM;
+        const int64_t wg96 = (N + 95) / 96 * m_tiles, wg48 = (N + 47) / 48 * m_tiles;
+        const int64_t cus = ctx->n_cu > 0 ? ctx->n_cu : 256;
+        const double cost96 = (double)((wg96 + cus - 1) / cus), cost48 = 0.65 * (double)((wg48 + cus - 1) / cus);
+        int tile_n = cost48 < cost96 ? 48 : 96;
+        if (ctx->gemm_tile_n == 48 || ctx->gemm_tile_n == 96) tile_n = ctx->gemm_tile_n;
+        const int32_t st = tile_n == 48 ? gemm_launch<48>(ctx, (const uint8_t *)W, Xh, Y, K, N, M)
+                                        : gemm_launch<96>(ctx, (const uint8_t *)W, Xh, Y, K, N, M);
+        if (st != GALOIS_HIP_OK) return st;
     } else {
         const dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
         hipLaunchKernelGGL(gemm_q4_0_mfma_v1, grid, dim3(256), 0, ctx->stream, (const uint8_t *)W, X, Y, K, N, M);
