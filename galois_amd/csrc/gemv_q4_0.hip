@@ -354,12 +354,14 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     // Every product's fields are fetched before any is chosen (the empty asm makes each an opaque value; left
     // alone, the compiler turns a select of two arguments into a second, dependent load from a selected address).
     int32_t k_blk0[MAXI], k_N[MAXI], k_ns[MAXI], k_groups[MAXI];
-    uint64_t k_W[MAXI], k_W2[MAXI], k_x[MAXI];  // pointers as bits: an address that has been through an asm is
-                                                // no longer known to be global memory and is cast back below
+    uint64_t k_W[MAXI], k_W2[MAXI], k_x[MAXI], k_nw[NORM ? MAXI : 1];  // pointers as bits: an address that has been
+                                                // through an asm is no longer known to be global memory and is cast back below
+    float k_eps[NORM ? MAXI : 1];
 #pragma unroll
     for (int k = 0; k < MAXI; k++) {
         k_blk0[k] = a.blk0[k], k_N[k] = a.N[k], k_ns[k] = a.nslots[k], k_groups[k] = a.groups[k];
         k_W[k] = (uint64_t)a.W[k], k_W2[k] = (uint64_t)a.W2[k], k_x[k] = (uint64_t)a.x[k];
+        if (NORM) k_nw[k] = (uint64_t)a.norm_w[k], k_eps[k] = a.eps[k];
     }
 #pragma unroll
     for (int k = 0; k < MAXI; k++) {
@@ -370,9 +372,14 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         asm volatile("" : "+s"(k_W[k]));
         asm volatile("" : "+s"(k_W2[k]));
         asm volatile("" : "+s"(k_x[k]));
+        if (NORM) {
+            asm volatile("" : "+s"(k_nw[k]));
+            asm volatile("" : "+s"(k_eps[k]));
+        }
     }
     int ii = 0, first_blk = 0;
-    uint64_t W_bits = k_W[0], W2_bits = k_W2[0], x_bits = k_x[0];
+    uint64_t W_bits = k_W[0], W2_bits = k_W2[0], x_bits = k_x[0], nw_bits = NORM ? k_nw[0] : 0;
+    float eps = NORM ? k_eps[0] : 0.0f;
     int N = k_N[0], ns = k_ns[0], groups = k_groups[0];
 #pragma unroll
     for (int k = 1; k < MAXI; k++) {
@@ -380,6 +387,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         ii = ge ? k : ii, first_blk = ge ? k_blk0[k] : first_blk;
         W_bits = ge ? k_W[k] : W_bits, W2_bits = ge ? k_W2[k] : W2_bits, x_bits = ge ? k_x[k] : x_bits;
         N = ge ? k_N[k] : N, ns = ge ? k_ns[k] : ns, groups = ge ? k_groups[k] : groups;
+        if (NORM) nw_bits = ge ? k_nw[k] : nw_bits, eps = ge ? k_eps[k] : eps;
     }
     typedef const __attribute__((address_space(1))) uint8_t *global_bytes;
     typedef const __attribute__((address_space(1))) float *global_floats;
@@ -403,12 +411,27 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     q4_slot q0[R];
     uint64_t dst_bits, res_bits;
     {
-        const float *wg = NORM ? a.norm_w[ii] : nullptr;
+        const float *wg = NORM ? (const float *)(global_floats)nw_bits : nullptr;
         float2 v[PG][4], nw[NORM ? PG : 1][4];
+        // Normalising preparation of a short vector (K <= 4096): the vector and the norm weight are fetched with
+        // fully coalesced 16-byte loads (a thread's eight values in weight-nibble order lie in four places, and
+        // fetching both arrays that way costs as much as a quarter of the weight stream), their product is staged
+        // in LDS behind the planes, and each thread gathers its eight values from there after the barrier the sum
+        // of squares needs anyway.
+        constexpr bool STAGED = NORM && PG == 1;
+        float4 sx[2], sg[2];
+        if (STAGED) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int i4 = min((int)threadIdx.x + j * THREADS, ns * 16 - 1);
+                sx[j] = reinterpret_cast<const float4 *>(xg)[i4];
+                sg[j] = reinterpret_cast<const float4 *>(wg)[i4];
+            }
+        }
 #pragma unroll
         for (int p = 0; p < PG; p++) {
             const int idx = threadIdx.x + p * THREADS;
-            if (idx < ns * 8) {
+            if (!STAGED && idx < ns * 8) {
                 const int slot = idx >> 3, g = idx & 7;
 #pragma unroll
                 for (int t = 0; t < 4; t += 2) {
@@ -440,26 +463,53 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         asm volatile("" : "+s"(res_bits));
         if (NORM) {
             float ss = 0.0f;
+            float *stage = reinterpret_cast<float *>(lds + ns * SD);
+            if (STAGED) {
 #pragma unroll
-            for (int p = 0; p < PG; p++)
-                if (threadIdx.x + p * THREADS < ns * 8) {
-#pragma unroll
-                    for (int t = 0; t < 4; t++) ss += v[p][t].x * v[p][t].x + v[p][t].y * v[p][t].y;
+                for (int j = 0; j < 2; j++) {
+                    const int i4 = (int)threadIdx.x + j * THREADS;
+                    if (i4 < ns * 16) {
+                        ss += sx[j].x * sx[j].x + sx[j].y * sx[j].y + sx[j].z * sx[j].z + sx[j].w * sx[j].w;
+                        reinterpret_cast<float4 *>(stage)[i4] =
+                            make_float4(sx[j].x * sg[j].x, sx[j].y * sg[j].y, sx[j].z * sg[j].z, sx[j].w * sg[j].w);
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int p = 0; p < PG; p++)
+                    if (threadIdx.x + p * THREADS < ns * 8) {
+#pragma unroll
+                        for (int t = 0; t < 4; t++) ss += v[p][t].x * v[p][t].x + v[p][t].y * v[p][t].y;
+                    }
+            }
             ss = wave_sum(ss);
             if (lane == 0) red[wave] = ss;
             __syncthreads();
             float tot = 0.0f;
 #pragma unroll
             for (int w = 0; w < WAVES; w++) tot += red[w];
-            const float inv = rsqrtf(tot / (float)(ns * 64) + a.eps[ii]);
+            const float inv = rsqrtf(tot / (float)(ns * 64) + eps);
+            if (STAGED) {
+                if ((int)threadIdx.x < ns * 8) {
+                    const int slot = threadIdx.x >> 3, g = threadIdx.x & 7;
 #pragma unroll
-            for (int p = 0; p < PG; p++)
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    v[p][t].x = (inv * v[p][t].x) * nw[NORM ? p : 0][t].x;
-                    v[p][t].y = (inv * v[p][t].y) * nw[NORM ? p : 0][t].y;
+                    for (int t = 0; t < 4; t += 2) {
+                        const int b = slot * 64 + xprep::group_x_index(g, 2 * t);
+                        const float2 lo = *reinterpret_cast<const float2 *>(stage + b);
+                        const float2 hi = *reinterpret_cast<const float2 *>(stage + b + 16);
+                        v[0][t] = make_float2(lo.x * inv, lo.y * inv);
+                        v[0][t + 1] = make_float2(hi.x * inv, hi.y * inv);
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int p = 0; p < PG; p++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        v[p][t].x = (inv * v[p][t].x) * nw[NORM ? p : 0][t].x;
+                        v[p][t].y = (inv * v[p][t].y) * nw[NORM ? p : 0][t].y;
+                    }
+            }
         }
 #pragma unroll
         for (int p = 0; p < PG; p++) {
@@ -592,7 +642,10 @@ void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, in
     constexpr int PGMAX = (kChunkSlots * 8 + WAVES * 64 - 1) / (WAVES * 64);
     constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
     if (max_slots <= 64) {
-        if (norm)
+        if (norm && PGSMALL == 1)  // room behind the planes for the staged, weighted activations (64 floats per slot)
+            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true, MAXI>), grid, block,
+                               lds + (size_t)max_slots * 64 * sizeof(float), ctx->stream, a);
+        else if (norm)
             hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true, MAXI>), grid, block, lds, ctx->stream, a);
         else
             hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, false, MAXI>), grid, block, lds, ctx->stream, a);
