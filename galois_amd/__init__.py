@@ -171,12 +171,15 @@ class Device:
     @staticmethod
     def gemv_items(items):
         """galois_hip_gemv_item array from dicts with vx, y, dst, ncols, nrows and optionally vx_up,
-        norm_weight, norm_eps, residual (build it once when the same launch is repeated)."""
+        norm_weight, norm_eps, residual, dst_scaled + scale_weight, sumsq_out, sumsq_in (build it once when the same
+        launch is repeated)."""
         arr = (_abi.GemvItem * max(1, len(items)))()
         for a, it in zip(arr, items):
             a.vx, a.y, a.dst = _ptr(it["vx"]), _ptr(it["y"]), _ptr(it["dst"])
             a.vx_up, a.norm_weight = _ptr(it.get("vx_up")), _ptr(it.get("norm_weight"))
             a.residual = _ptr(it.get("residual"))
+            a.dst_scaled, a.scale_weight = _ptr(it.get("dst_scaled")), _ptr(it.get("scale_weight"))
+            a.sumsq_out, a.sumsq_in = _ptr(it.get("sumsq_out")), _ptr(it.get("sumsq_in"))
             a.ncols, a.nrows, a.norm_eps = it["ncols"], it["nrows"], it.get("norm_eps", 0.0)
         arr.n_items = len(items)
         return arr

@@ -17,7 +17,8 @@ sz = C.c_size_t
 class GemvItem(C.Structure):
     """galois_hip_gemv_item of include/galois_hip.h, field for field."""
     _fields_ = [("vx", vp), ("vx_up", vp), ("y", vp), ("norm_weight", vp), ("residual", vp), ("dst", vp),
-                ("ncols", i32), ("nrows", i32), ("norm_eps", f32)]
+                ("ncols", i32), ("nrows", i32), ("norm_eps", f32), ("reserved", i32), ("dst_scaled", vp),
+                ("scale_weight", vp), ("sumsq_out", vp), ("sumsq_in", vp)]
 
 
 # name -> (restype, argtypes); must list every function the header declares

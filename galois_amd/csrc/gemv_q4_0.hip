@@ -332,21 +332,34 @@ struct gg_args {
     int32_t N[GG_MAX];
     int32_t nslots[GG_MAX];
     int32_t groups[GG_MAX];       // row groups a wave works through, one after the other
-    const float *norm_w[GG_MAX];  // RMSNorm weight or null
+    const float *norm_w[GG_MAX];  // NORM 1: RMSNorm weight; NORM 2: the partial sums of squares of the activations
     float *dst[GG_MAX];
     const float *residual[GG_MAX];  // or null
     float eps[GG_MAX];
+    float *dst2[GG_MAX];          // OUT2: second copy of the result, multiplied by scale2, or null
+    const float *scale2[GG_MAX];
+    float *ssq_out[GG_MAX];       // OUT2: sum of squares of the result, one float per workgroup (16 rows), or null
 };
 
 // A wave owns R slots per lane: R rows, or R / 2 rows of a gate / up pair; a workgroup WAVES times that.
-// PG: activation groups (8 values) one thread prepares at most; NORM: the vector is normalised first.
+// PG: activation groups (8 values) one thread prepares at most.
+// NORM 1: the vector is normalised (rms_norm) and multiplied by a weight first.  NORM 2: the vector arrives already
+// multiplied by the weight and the sums of squares of the unweighted vector arrive as per-16-row partials (written
+// by the launch that produced the vector, OUT2): w . (inv * xg) = inv * (w . xg), so the product runs on the vector as
+// it is and the result is multiplied by inv = rsqrt(mean + eps) at the end -- no second vector to fetch and no
+// barrier before the preparation.
+// OUT2: the launch also writes result * scale2 and the workgroup's sum of squares of the result.
 // MAXI: products the selects look at (4 keeps all of their operands in scalar registers at once).
-template <int L, int R, int WAVES, int PG, int OCC, bool NORM, int MAXI>
+template <int L, int R, int WAVES, int PG, int OCC, int NORM_MODE, int MAXI, bool OUT2>
 __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     __shared__ float red[WAVES];
+    __shared__ float red2[WAVES];
     constexpr int SD = slot_lds<L>::dwords;
     constexpr int THREADS = WAVES * 64;
+    constexpr bool NORM = NORM_MODE == 1;    // normalise here
+    constexpr bool NORM2 = NORM_MODE == 2;   // scale the result by inv from the partial sums of squares
+    constexpr bool NARG = NORM_MODE != 0;    // the norm_w / eps arguments are used
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     GH_TSTAMP(0);
@@ -354,14 +367,14 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     // Every product's fields are fetched before any is chosen (the empty asm makes each an opaque value; left
     // alone, the compiler turns a select of two arguments into a second, dependent load from a selected address).
     int32_t k_blk0[MAXI], k_N[MAXI], k_ns[MAXI], k_groups[MAXI];
-    uint64_t k_W[MAXI], k_W2[MAXI], k_x[MAXI], k_nw[NORM ? MAXI : 1];  // pointers as bits: an address that has been
+    uint64_t k_W[MAXI], k_W2[MAXI], k_x[MAXI], k_nw[NARG ? MAXI : 1];  // pointers as bits: an address that has been
                                                 // through an asm is no longer known to be global memory and is cast back below
-    float k_eps[NORM ? MAXI : 1];
+    float k_eps[NARG ? MAXI : 1];
 #pragma unroll
     for (int k = 0; k < MAXI; k++) {
         k_blk0[k] = a.blk0[k], k_N[k] = a.N[k], k_ns[k] = a.nslots[k], k_groups[k] = a.groups[k];
         k_W[k] = (uint64_t)a.W[k], k_W2[k] = (uint64_t)a.W2[k], k_x[k] = (uint64_t)a.x[k];
-        if (NORM) k_nw[k] = (uint64_t)a.norm_w[k], k_eps[k] = a.eps[k];
+        if (NARG) k_nw[k] = (uint64_t)a.norm_w[k], k_eps[k] = a.eps[k];
     }
 #pragma unroll
     for (int k = 0; k < MAXI; k++) {
@@ -372,14 +385,14 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         asm volatile("" : "+s"(k_W[k]));
         asm volatile("" : "+s"(k_W2[k]));
         asm volatile("" : "+s"(k_x[k]));
-        if (NORM) {
+        if (NARG) {
             asm volatile("" : "+s"(k_nw[k]));
             asm volatile("" : "+s"(k_eps[k]));
         }
     }
     int ii = 0, first_blk = 0;
-    uint64_t W_bits = k_W[0], W2_bits = k_W2[0], x_bits = k_x[0], nw_bits = NORM ? k_nw[0] : 0;
-    float eps = NORM ? k_eps[0] : 0.0f;
+    uint64_t W_bits = k_W[0], W2_bits = k_W2[0], x_bits = k_x[0], nw_bits = NARG ? k_nw[0] : 0;
+    float eps = NARG ? k_eps[0] : 0.0f;
     int N = k_N[0], ns = k_ns[0], groups = k_groups[0];
 #pragma unroll
     for (int k = 1; k < MAXI; k++) {
@@ -387,7 +400,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         ii = ge ? k : ii, first_blk = ge ? k_blk0[k] : first_blk;
         W_bits = ge ? k_W[k] : W_bits, W2_bits = ge ? k_W2[k] : W2_bits, x_bits = ge ? k_x[k] : x_bits;
         N = ge ? k_N[k] : N, ns = ge ? k_ns[k] : ns, groups = ge ? k_groups[k] : groups;
-        if (NORM) nw_bits = ge ? k_nw[k] : nw_bits, eps = ge ? k_eps[k] : eps;
+        if (NARG) nw_bits = ge ? k_nw[k] : nw_bits, eps = ge ? k_eps[k] : eps;
     }
     typedef const __attribute__((address_space(1))) uint8_t *global_bytes;
     typedef const __attribute__((address_space(1))) float *global_floats;
@@ -409,7 +422,8 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     // are requested first and the first weights right behind them: the preparation then runs while the weights
     // are in flight.
     q4_slot q0[R];
-    uint64_t dst_bits, res_bits;
+    uint64_t dst_bits, res_bits, dst2_bits = 0, scale2_bits = 0, ssq_bits = 0;
+    float scale2_first = 0.0f;
     {
         const float *wg = NORM ? (const float *)(global_floats)nw_bits : nullptr;
         float2 v[PG][4], nw[NORM ? PG : 1][4];
@@ -445,6 +459,16 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                 }
             }
         }
+        float psq = 0.0f;
+        if (NORM2) {  // one partial per 16 elements of the vector: ns * 4 of them
+            const float *sq = (const float *)(global_floats)nw_bits;
+            constexpr int PQ = (GG_MAX_SLOTS * 4 + THREADS - 1) / THREADS;
+            float t[PQ];
+#pragma unroll
+            for (int p = 0; p < PQ; p++) t[p] = sq[min((int)threadIdx.x + p * THREADS, ns * 4 - 1)];
+#pragma unroll
+            for (int p = 0; p < PQ; p++) psq += (int)threadIdx.x + p * THREADS < ns * 4 ? t[p] : 0.0f;
+        }
         // q[j] = slot `lane` of row row0 + j of W; for a gate / up pair q[j] = row row0 + j of W (j < R/2) or of W2.
         // Rows past N are loaded from row N - 1 and never stored.
         {
@@ -461,6 +485,20 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         dst_bits = (uint64_t)a.dst[ii], res_bits = (uint64_t)a.residual[ii];
         asm volatile("" : "+s"(dst_bits));
         asm volatile("" : "+s"(res_bits));
+        if (OUT2) {
+            dst2_bits = (uint64_t)a.dst2[ii], scale2_bits = (uint64_t)a.scale2[ii], ssq_bits = (uint64_t)a.ssq_out[ii];
+            asm volatile("" : "+s"(dst2_bits));
+            asm volatile("" : "+s"(scale2_bits));
+            asm volatile("" : "+s"(ssq_bits));
+        }
+        if (OUT2) {  // the first group's scale values ride behind the weights (always a load: see the activations)
+            const float *sp = scale2_bits ? (const float *)(global_floats)scale2_bits + min(row0 + (lane < rw ? lane : 0), N - 1) : xg;
+            scale2_first = *sp;
+        }
+        if (NORM2) {  // the partial sums reach every wave through the barrier that publishes the planes
+            psq = wave_sum(psq);
+            if (lane == 0) red[wave] = psq;
+        }
         if (NORM) {
             float ss = 0.0f;
             float *stage = reinterpret_cast<float *>(lds + ns * SD);
@@ -537,6 +575,15 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     GH_TSTAMP(3);
     __syncthreads();
     GH_TSTAMP(4);
+    float inv2 = 1.0f;
+    if (NORM2) {
+        float tot = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) tot += red[w];
+        // the same value in every lane: kept in a scalar register (the kernel has no vector register to spare)
+        inv2 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrtf(tot / (float)(ns * 64) + eps))));
+    }
+    float sq_out = 0.0f;  // OUT2: squares of this lane's results
 
     // One group of rows.  The first group's first slots are the ones requested before the preparation; it is
     // peeled off the loop so that those registers are not kept alive through the later groups.
@@ -586,6 +633,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                 float gt = wave_sum_to_lane63(acc[j]), up = wave_sum_to_lane63(acc[R / 2 + j]);
                 gt = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gt), 63));
                 up = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, up), 63));
+                if (NORM2) gt *= inv2, up *= inv2;
                 if (lane == j) out = gt / (1.0f + expf(-gt)) * up;
             }
         } else {
@@ -593,6 +641,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             for (int j = 0; j < R; j++) {
                 float t = wave_sum_to_lane63(acc[j]);
                 t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
+                if (NORM2) t *= inv2;
                 if (lane == j) out = t;
             }
         }
@@ -601,6 +650,12 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             const float *res = (const float *)(global_floats)res_bits;
             if (res) out += res[row0 + lane];
             ((float *)(global_out)dst_bits)[row0 + lane] = out;
+            if (OUT2) {
+                if (dst2_bits)
+                    ((float *)(global_out)dst2_bits)[row0 + lane] =
+                        out * (FIRST ? scale2_first : ((const float *)(global_floats)scale2_bits)[row0 + lane]);
+                sq_out = __builtin_fmaf(out, out, sq_out);
+            }
         }
 #pragma unroll
         for (int j = 0; j < R; j++) acc[j] = 0.0f;
@@ -610,6 +665,18 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         row0 += WAVES * rw;
         if (row0 >= N) break;  // wave-uniform
         do_group(std::false_type{});
+    }
+    if (OUT2 && ssq_bits) {  // wave-uniform; every wave of the workgroup gets here
+        sq_out = wave_sum(sq_out);
+        if (lane == 0) red2[wave] = sq_out;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float tot = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WAVES; w++) tot += red2[w];
+            typedef __attribute__((address_space(1))) float *global_out;
+            ((float *)(global_out)ssq_bits)[(int)blockIdx.x - first_blk] = tot;
+        }
     }
     GH_TSTAMP(6);
 }
@@ -635,35 +702,47 @@ void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst
 }
 
 // Host side of the group kernel: checks, the block range of every matrix, launch.
+// mode: 0 plain, 1 normalising, 2 pre-weighted activations + partial sums of squares; out2: second outputs.
+// The second outputs exist for plain launches of at most four products (what produces a residual stream).
 template <int L, int R, int WAVES, int OCC, int MAXI>
-void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, int max_slots, bool norm) {
+void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, int max_slots, int mode, bool out2) {
     const dim3 grid(blocks), block(WAVES * 64);
     const size_t lds = (size_t)max_slots * slot_lds<L>::dwords * sizeof(uint32_t);
     constexpr int PGMAX = (kChunkSlots * 8 + WAVES * 64 - 1) / (WAVES * 64);
     constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
+    constexpr int OCCN = OCC > 4 ? 4 : OCC;  // the normalising preparation of a long vector needs more than 64 registers
+#define GG_LAUNCH(PG_, OCC_, MODE_, OUT2_, LDS_) \
+    hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PG_, OCC_, MODE_, MAXI, OUT2_>), grid, block, LDS_, ctx->stream, a)
     if (max_slots <= 64) {
-        if (norm && PGSMALL == 1)  // room behind the planes for the staged, weighted activations (64 floats per slot)
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true, MAXI>), grid, block,
-                               lds + (size_t)max_slots * 64 * sizeof(float), ctx->stream, a);
-        else if (norm)
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, true, MAXI>), grid, block, lds, ctx->stream, a);
+        if (mode == 1 && PGSMALL == 1)  // room behind the planes for the staged, weighted activations (64 floats per slot)
+            GG_LAUNCH(PGSMALL, OCC, 1, false, lds + (size_t)max_slots * 64 * sizeof(float));
+        else if (mode == 1)
+            GG_LAUNCH(PGSMALL, OCC, 1, false, lds);
+        else if (mode == 2)
+            GG_LAUNCH(PGSMALL, OCC, 2, false, lds);
+        else if (out2 && MAXI == 4)
+            GG_LAUNCH(PGSMALL, OCC, 0, (MAXI == 4), lds);
         else
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, false, MAXI>), grid, block, lds, ctx->stream, a);
+            GG_LAUNCH(PGSMALL, OCC, 0, false, lds);
     } else {
-        if (norm)  // the normalising preparation of a long vector needs more than 64 registers
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, (OCC > 4 ? 4 : OCC), true, MAXI>), grid, block, lds,
-                               ctx->stream, a);
+        if (mode == 1)
+            GG_LAUNCH(PGMAX, OCCN, 1, false, lds);
+        else if (mode == 2)
+            GG_LAUNCH(PGMAX, OCC, 2, false, lds);
+        else if (out2 && MAXI == 4)
+            GG_LAUNCH(PGMAX, OCC, 0, (MAXI == 4), lds);
         else
-            hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGMAX, OCC, false, MAXI>), grid, block, lds, ctx->stream, a);
+            GG_LAUNCH(PGMAX, OCC, 0, false, lds);
     }
+#undef GG_LAUNCH
 }
 
 template <int L, int R, int WAVES, int OCC>
-void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, int n_items, unsigned blocks, int max_slots, bool norm) {
+void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, int n_items, unsigned blocks, int max_slots, int mode, bool out2) {
     if (n_items <= 4)
-        launch_group_cfg<L, R, WAVES, OCC, 4>(ctx, a, blocks, max_slots, norm);
+        launch_group_cfg<L, R, WAVES, OCC, 4>(ctx, a, blocks, max_slots, mode, out2);
     else
-        launch_group_cfg<L, R, WAVES, OCC, GG_MAX>(ctx, a, blocks, max_slots, norm);
+        launch_group_cfg<L, R, WAVES, OCC, GG_MAX>(ctx, a, blocks, max_slots, mode, out2);
 }
 
 int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what) {
@@ -673,7 +752,8 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     memset(&a, 0, sizeof(a));
     int32_t max_slots = 0;
     int64_t rows = 0;
-    bool norm = false;
+    int mode = 0;      // 0 plain, 1 normalising, 2 pre-weighted activations + partial sums of squares
+    bool out2 = false;
     for (int i = 0; i < GG_MAX; i++) a.blk0[i] = 0x7FFFFFFF;
     for (int i = 0; i < n_items; i++) {
         const galois_hip_gemv_item &s = items[i];
@@ -683,11 +763,26 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
         GH_REQUIRE(ctx, gh_aligned(s.vx, 4) && gh_aligned(s.vx_up, 4) && gh_aligned(s.y, 8) && gh_aligned(s.norm_weight, 8) &&
                             gh_aligned(s.residual, 4) && gh_aligned(s.dst, 4),
                    GALOIS_HIP_E_ALIGN, "gemv group: matrices 4-byte, activations and norm weights 8-byte, vectors 4-byte aligned");
-        if (i == 0) norm = s.norm_weight != nullptr;
-        GH_REQUIRE(ctx, (s.norm_weight != nullptr) == norm, GALOIS_HIP_E_UNSUPPORTED,
-                   "gemv group: either every product of a call normalises its activations or none does");
+        GH_REQUIRE(ctx, !(s.norm_weight && s.sumsq_in), GALOIS_HIP_E_UNSUPPORTED,
+                   "gemv group: norm_weight (normalise here) and sumsq_in (activations already weighted) exclude each other");
+        const int m = s.norm_weight ? 1 : (s.sumsq_in ? 2 : 0);
+        if (i == 0) mode = m;
+        GH_REQUIRE(ctx, m == mode, GALOIS_HIP_E_UNSUPPORTED,
+                   "gemv group: the products of a call all normalise their activations the same way or not at all");
+        GH_REQUIRE(ctx, (s.dst_scaled == nullptr) == (s.scale_weight == nullptr), GALOIS_HIP_E_NULL,
+                   "gemv group: dst_scaled and scale_weight go together");
+        if (s.dst_scaled || s.sumsq_out) {
+            GH_REQUIRE(ctx, m == 0 && !s.vx_up && n_items <= 4 && ctx->gemv_units_per_wave <= 1, GALOIS_HIP_E_UNSUPPORTED,
+                       "gemv group: dst_scaled / sumsq_out are written by plain products (no norm, no pair) in calls of at most four");
+            GH_REQUIRE(ctx, gh_aligned(s.dst_scaled, 4) && gh_aligned(s.scale_weight, 4) && gh_aligned(s.sumsq_out, 4),
+                       GALOIS_HIP_E_ALIGN, "gemv group: 4-byte aligned vectors");
+            out2 = true;
+        }
+        GH_REQUIRE(ctx, gh_aligned(s.sumsq_in, 4), GALOIS_HIP_E_ALIGN, "gemv group: 4-byte aligned vectors");
         a.W[i] = (const uint8_t *)s.vx, a.W2[i] = (const uint8_t *)s.vx_up, a.dst[i] = s.dst, a.residual[i] = s.residual;
-        a.x[i] = s.y, a.norm_w[i] = s.norm_weight, a.eps[i] = s.norm_eps, a.N[i] = s.nrows, a.nslots[i] = s.ncols / 64;
+        a.x[i] = s.y, a.norm_w[i] = m == 2 ? s.sumsq_in : s.norm_weight, a.eps[i] = s.norm_eps, a.N[i] = s.nrows;
+        a.nslots[i] = s.ncols / 64;
+        a.dst2[i] = s.dst_scaled, a.scale2[i] = s.scale_weight, a.ssq_out[i] = s.sumsq_out;
         if (a.nslots[i] > max_slots) max_slots = a.nslots[i];
         rows += (int64_t)s.nrows * (s.vx_up ? 2 : 1);
     }
@@ -714,11 +809,11 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     }
     GH_BIND(ctx);
     if (cfg == 1)
-        launch_group_cfg<5, 1, 16, 4>(ctx, a, n_items, (unsigned)blocks, max_slots, norm);
+        launch_group_cfg<5, 1, 16, 4>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
     else if (cfg == 7)
-        launch_group_cfg<5, 2, 8, 8>(ctx, a, n_items, (unsigned)blocks, max_slots, norm);
+        launch_group_cfg<5, 2, 8, 8>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
     else
-        launch_group_cfg<5, 2, 8, 6>(ctx, a, n_items, (unsigned)blocks, max_slots, norm);
+        launch_group_cfg<5, 2, 8, 6>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
     GH_LAUNCH_CHECK(ctx, what);
 }
 

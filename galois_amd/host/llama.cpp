@@ -1,6 +1,8 @@
 // LLaMA decode step over the galois op mirror (see llama.hpp).
 #include "llama.hpp"
 
+#include <cstring>
+
 #include <cmath>
 
 namespace galois {
@@ -41,11 +43,13 @@ GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst) {
 GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
     if (items.empty() || items.size() > 8) return err(GError::ShapeError, "galois_matvec_group: 1 to 8 products");
     galois_hip_gemv_item it[8];
+    memset(it, 0, sizeof(it));
     std::shared_ptr<CudaDevice> dev;
     for (size_t i = 0; i < items.size(); i++) {
         const MatvecItem &m = items[i];
         if (!m.w || !m.x || !m.dst) return err(GError::Unexpected, "galois_matvec_group: w, x and dst are required");
-        for (const Tensor *t : {m.w, m.w_up, m.x, m.norm_weight, m.residual, (const Tensor *)m.dst}) {
+        for (const Tensor *t : {m.w, m.w_up, m.x, m.norm_weight, m.residual, (const Tensor *)m.dst, (const Tensor *)m.dst_scaled,
+                                m.scale_weight, (const Tensor *)m.sumsq_out, m.sumsq_in}) {
             if (!t) continue;
             if (!t->device().is_gpu()) return err(GError::Unimplemented, "galois_matvec_group: Gpu tensors only");
             if (!dev) dev = t->device().gpu;
@@ -54,13 +58,21 @@ GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
         }
         if (m.w->dtype() != GGmlType::Q4_0 || (m.w_up && m.w_up->dtype() != GGmlType::Q4_0))
             return err(GError::Unimplemented, "galois_matvec_group: Q4_0 matrices only");
-        for (const Tensor *t : {m.x, m.norm_weight, m.residual, (const Tensor *)m.dst})
+        for (const Tensor *t : {m.x, m.norm_weight, m.residual, (const Tensor *)m.dst, (const Tensor *)m.dst_scaled, m.scale_weight,
+                                (const Tensor *)m.sumsq_out, m.sumsq_in})
             if (t && t->dtype() != GGmlType::F32) return err(GError::Unimplemented, "galois_matvec_group: F32 vectors only");
         const size_t K = m.w->dim().shape[0], N = m.w->dim().shape[1];
         if (m.w->dim().elem_count() != K * N || m.x->dim().elem_count() != K || m.dst->dim().elem_count() != N ||
             (m.w_up && (m.w_up->dim().shape[0] != K || m.w_up->dim().elem_count() != K * N)) ||
             (m.norm_weight && m.norm_weight->dim().elem_count() != K) || (m.residual && m.residual->dim().elem_count() != N))
             return err(GError::ShapeError, "galois_matvec_group: w [K, N], w_up [K, N], x and norm_weight K, dst and residual N elements");
+        if ((m.dst_scaled && m.dst_scaled->dim().elem_count() != N) || (m.scale_weight && m.scale_weight->dim().elem_count() != N) ||
+            (m.sumsq_out && m.sumsq_out->dim().elem_count() < (N + 15) / 16) || (m.sumsq_in && m.sumsq_in->dim().elem_count() < (K + 15) / 16))
+            return err(GError::ShapeError, "galois_matvec_group: dst_scaled and scale_weight N elements, sumsq_out ceil(N / 16), sumsq_in ceil(K / 16)");
+        it[i].dst_scaled = m.dst_scaled ? (float *)m.dst_scaled->data() : nullptr;
+        it[i].scale_weight = m.scale_weight ? (const float *)m.scale_weight->data() : nullptr;
+        it[i].sumsq_out = m.sumsq_out ? (float *)m.sumsq_out->data() : nullptr;
+        it[i].sumsq_in = m.sumsq_in ? (const float *)m.sumsq_in->data() : nullptr;
         it[i].vx = m.w->data(), it[i].vx_up = m.w_up ? m.w_up->data() : nullptr, it[i].y = (const float *)m.x->data();
         it[i].norm_weight = m.norm_weight ? (const float *)m.norm_weight->data() : nullptr;
         it[i].residual = m.residual ? (const float *)m.residual->data() : nullptr;
@@ -143,6 +155,8 @@ GResult LlamaDecoder::create(const LlamaHParams &hp, const Device &dev, std::uni
     G_TRY(mk(&m->o_, F32, dev, D, 1, H));
     for (Tensor *t : {&m->g_, &m->u_, &m->h_}) G_TRY(mk(t, F32, dev, F, 1));
     G_TRY(mk(&m->logits_, F32, dev, V, 1));
+    G_TRY(mk(&m->ssq_, F32, dev, (E + 15) / 16));
+    G_TRY(mk(&m->ssq1_, F32, dev, (E + 15) / 16));
     *out = std::move(m);
     return GError{};
 }
@@ -212,9 +226,16 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
         return m;
     };
     for (Layer &l : layers_) {
+        const size_t li = (size_t)(&l - &layers_[0]);
+        const bool split = fused >= 4;       // norms split over producer and consumer launches
         if (grouped) {  // rms_norm * weight + the three projections: one launch
             MatvecItem mq = item(l.wq, x_, q_), mk_ = item(l.wk, x_, k_), mv = item(l.wv, x_, v_);
-            mq.norm_weight = mk_.norm_weight = mv.norm_weight = &l.attn_norm;
+            if (split && li > 0) {  // the previous layer's last launch left x * attn_norm in a_ and the sums of squares of x
+                mq.x = mk_.x = mv.x = &a_;
+                mq.sumsq_in = mk_.sumsq_in = mv.sumsq_in = &ssq_;
+            } else {
+                mq.norm_weight = mk_.norm_weight = mv.norm_weight = &l.attn_norm;
+            }
             G_TRY(galois_matvec_group({mq, mk_, mv})); ops++;
         } else {
             G_TRY(norm(x_, l.attn_norm, a_));
@@ -227,12 +248,19 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
             ops++;
             MatvecItem mo = item(l.wo, ao_, x1_);
             mo.residual = &x_;
+            if (split) mo.dst_scaled = &f_, mo.scale_weight = &l.ffn_norm, mo.sumsq_out = &ssq1_;
             G_TRY(galois_matvec_group({mo})); ops++;
-            MatvecItem mg = item(l.w_gate, x1_, h_);
-            mg.w_up = &l.w_up, mg.norm_weight = &l.ffn_norm;
+            MatvecItem mg = item(l.w_gate, split ? f_ : x1_, h_);
+            mg.w_up = &l.w_up;
+            if (split)
+                mg.sumsq_in = &ssq1_;
+            else
+                mg.norm_weight = &l.ffn_norm;
             G_TRY(galois_matvec_group({mg})); ops++;
             MatvecItem md = item(l.w_down, h_, x_);
             md.residual = &x1_;
+            if (split)  // x times the weight of the norm that reads it next: the next layer's, or the output norm
+                md.dst_scaled = &a_, md.scale_weight = li + 1 < layers_.size() ? &layers_[li + 1].attn_norm : &out_norm_, md.sumsq_out = &ssq_;
             G_TRY(galois_matvec_group({md})); ops++;
             continue;
         }
@@ -291,7 +319,10 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
     }
     if (grouped) {
         MatvecItem ml = item(output_, x_, logits_);
-        ml.norm_weight = &out_norm_;
+        if (fused >= 4)
+            ml.x = &a_, ml.sumsq_in = &ssq_;
+        else
+            ml.norm_weight = &out_norm_;
         G_TRY(galois_matvec_group({ml})); ops++;
     } else {
         G_TRY(norm(x_, out_norm_, a_));

@@ -37,8 +37,11 @@ class LlamaDecoder {
     // rms_norm*weight and silu*up kernels instead of two ops each.
     // fused = 2 additionally sends the Q4_0 matrix-vector products out in grouped launches (q | k | v together,
     // gate | up as a SwiGLU pair) with the norms, silu * up and the residual adds riding along: 12 launches per layer;
-    // fused = 3 also replaces the eight attention ops of a layer by galois_attn_decode: 5 launches per layer
-    // (the only plan that runs with an f16 KV cache).
+    // fused = 3 also replaces the eight attention ops of a layer by galois_attn_decode: 5 launches per layer;
+    // fused = 4 splits the norms that follow a residual add over the launch that produces the residual stream (it
+    // also writes the stream times the next norm weight and its partial sums of squares) and the launch that consumes
+    // it (it fetches one vector instead of two and waits for no reduction): the same 5 launches per layer.
+    // fused >= 3 are the plans that run with an f16 KV cache.
     GResult decode(int32_t token, int32_t n_past, int fused);
     // Records the same step as a graph / replays the recorded step.
     GResult capture(int32_t token, int32_t n_past, int fused);
@@ -60,6 +63,7 @@ class LlamaDecoder {
     std::vector<Layer> layers_;
     Tensor tok_id_, pos_, scale_;                                    // I32 [1], I32 [1], host f32 [1]
     Tensor x_, t_, a_, q_, k_, v_, qr_, kr_, s_, p_, o_, ao_, x1_, f_, g_, u_, h_, d_, logits_;
+    Tensor ssq_, ssq1_;  // partial sums of squares of x and x1 (fused = 4)
     galois_hip_graph *graph_ = nullptr;
     size_t n_ops_ = 0;
     int32_t last_token_ = -1, last_pos_ = -1;
@@ -73,10 +77,15 @@ GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst);
 // Several Q4_0 matrix-vector products in one launch (galois_hip_dequantize_mul_mat_vec_q4_0_group): per product
 // dst = w . x, where x is first replaced by rms_norm(x, eps) * norm_weight when norm_weight is set, the result
 // becomes silu(w . x) * (w_up . x) when w_up is set, and residual is added when set (it may be dst).
+// A norm can be split over two calls: the call that produces a vector also writes dst_scaled = dst * scale_weight and
+// sumsq_out (the sums of squares of dst per 16 elements); the call that consumes it passes x = that dst_scaled,
+// sumsq_in = that sumsq_out and eps, and gets w . (rms_norm(dst, eps) * scale_weight) up to rounding.
 struct MatvecItem {
     const Tensor *w = nullptr, *w_up = nullptr, *x = nullptr, *norm_weight = nullptr, *residual = nullptr;
     Tensor *dst = nullptr;
     float eps = 0.0f;
+    Tensor *dst_scaled = nullptr, *sumsq_out = nullptr;
+    const Tensor *scale_weight = nullptr, *sumsq_in = nullptr;
 };
 GResult galois_matvec_group(const std::vector<MatvecItem> &items);
 

@@ -129,10 +129,19 @@ int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, const void *
  *     src/cuda.rs:1665-1688, 1190-1215); vx_up has the shape of vx;
  *   residual != NULL: residual[row] is added to the result (add_f32, src/cuda.rs:1188-1244);
  *     residual may be dst.
+ * A normalisation can also be split over two launches, so that the second fetches one vector instead of two and
+ * waits for no reduction: the launch that produces a vector x (a plain product, usually with a residual) also writes
+ *   dst_scaled[row] = dst[row] * scale_weight[row]  (x times the weight of the norm that follows), and
+ *   sumsq_out[row / 16] = sum of dst[row]^2 over the 16 rows, ceil(nrows / 16) floats;
+ * the launch that consumes it passes y = that dst_scaled and sumsq_in = that sumsq_out (ceil(ncols / 16) floats)
+ * with norm_eps, and computes (vx . y) * rsqrt(sum(sumsq_in) / ncols + norm_eps), which is
+ * vx . (rms_norm(x, norm_eps) * weight) up to rounding (the scalar is applied to both products of a pair).
+ * dst_scaled and scale_weight go together; dst_scaled / sumsq_out need norm_weight, sumsq_in and vx_up NULL and at
+ * most four products in the call; norm_weight and sumsq_in exclude each other.
  * Each product is what galois_hip_dequantize_mul_mat_vec_q4_0 computes.  1 <= n_items <= 8;
  * ncols % 64 == 0 and ncols <= 12288; matrices 4-byte aligned, y and norm_weight 8-byte aligned;
- * either every product of a call has a norm_weight or none has.  The items array is read during
- * the call only. */
+ * the products of a call all have a norm_weight, or all a sumsq_in, or none has either.  The items array is
+ * read during the call only; unused pointer fields are NULL. */
 typedef struct galois_hip_gemv_item {
     const void *vx;
     const void *vx_up;
@@ -142,6 +151,11 @@ typedef struct galois_hip_gemv_item {
     float *dst;
     int32_t ncols, nrows;
     float norm_eps;
+    int32_t reserved;  /* 0 */
+    float *dst_scaled;
+    const float *scale_weight;
+    float *sumsq_out;
+    const float *sumsq_in;
 } galois_hip_gemv_item;
 int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items,
                                                      int32_t n_items);

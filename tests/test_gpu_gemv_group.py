@@ -170,6 +170,52 @@ def test_group_of_six_with_norm_pairs_and_residuals(dev):
         _check(got, _ref_item(it), i)
 
 
+@pytest.mark.parametrize("k,n1,n2", [(4096, 4096, 11008), (256, 100, 33), (11008, 4096, 300), (64, 17, 5)])
+def test_group_norm_split_over_two_launches(dev, k, n1, n2):
+    """A launch that produces a vector also writes it times the next norm's weight and its sums of squares per 16
+    rows; the next launch consumes those instead of normalising: same result as normalising in the second launch."""
+    rng = np.random.default_rng(k + n1)
+    h = rng.standard_normal(k).astype(np.float32)
+    res = rng.standard_normal(n1).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(n1)).astype(np.float32)
+    w1, w2, w2u = _wx(1, k, n1), _wx(2, n1, n2) if n1 % 64 == 0 else None, None
+    eps = 1e-5
+    b = {name: dev.upload(a) for name, a in (("h", h), ("res", res), ("g", g), ("w1", w1))}
+    x, xs, sq = dev.alloc(n1 * 4), dev.alloc(n1 * 4), dev.alloc(((n1 + 15) // 16) * 4 + 64)
+    dev.upload(np.full((n1 + 15) // 16 + 16, 7.5, np.float32), sq)
+    dev.dequantize_mul_mat_vec_q4_0_group([{"vx": b["w1"], "y": b["h"], "dst": x, "ncols": k, "nrows": n1,
+                                            "residual": b["res"], "dst_scaled": xs, "scale_weight": b["g"],
+                                            "sumsq_out": sq}])
+    x_ref = _ref_item({"vx": w1, "y": h, "residual": res})
+    x_g = dev.download(x, np.float32, n1)
+    _check(x_g, x_ref, "x")
+    np.testing.assert_array_equal(dev.download(xs, np.float32, n1), x_g * g)        # one f32 product per element
+    sq_g = dev.download(sq, np.float32, (n1 + 15) // 16 + 16)
+    assert np.all(sq_g[(n1 + 15) // 16:] == 7.5), "wrote past the end of sumsq_out"
+    pad = np.zeros(((n1 + 15) // 16) * 16)
+    pad[:n1] = x_g.astype(np.float64) ** 2
+    np.testing.assert_allclose(sq_g[:(n1 + 15) // 16], pad.reshape(-1, 16).sum(1), rtol=1e-5)
+    if w2 is not None:   # the consuming launch, plain and as a SwiGLU pair, against normalising there
+        w2u = _wx(3, n1, n2)
+        bw2, bw2u = dev.upload(w2), dev.upload(w2u)
+        y_split, y_norm, p_split = dev.alloc(n2 * 4), dev.alloc(n2 * 4), dev.alloc(n2 * 4)
+        dev.dequantize_mul_mat_vec_q4_0_group([{"vx": bw2, "y": xs, "dst": y_split, "ncols": n1, "nrows": n2,
+                                                "sumsq_in": sq, "norm_eps": eps},
+                                               {"vx": bw2, "vx_up": bw2u, "y": xs, "dst": p_split, "ncols": n1,
+                                                "nrows": n2, "sumsq_in": sq, "norm_eps": eps}])
+        dev.dequantize_mul_mat_vec_q4_0_group([{"vx": bw2, "y": x, "dst": y_norm, "ncols": n1, "nrows": n2,
+                                                "norm_weight": b["g"], "norm_eps": eps}])
+        ref = _ref_item({"vx": w2, "y": x_g, "norm_weight": g, "norm_eps": eps})
+        _check(dev.download(y_split, np.float32, n2), ref, "split")
+        _check(dev.download(y_norm, np.float32, n2), ref, "norm")
+        _check(dev.download(p_split, np.float32, n2), _ref_item({"vx": w2, "vx_up": w2u, "y": x_g, "norm_weight": g,
+                                                                 "norm_eps": eps}), "split pair")
+        for t in (bw2, bw2u, y_split, y_norm, p_split):
+            dev.free(t)
+    for t in list(b.values()) + [x, xs, sq]:
+        dev.free(t)
+
+
 def test_group_special_values(dev):
     k, n = 4096, 40
     wq = _wx(99, k, n)
@@ -180,6 +226,20 @@ def test_group_special_values(dev):
         got, other = _run_group(dev, [{"vx": wq, "y": e}, {"vx": wq, "y": np.ones(k, np.float32)}])
         assert np.array_equal(got, w[:, kk])
         _check(other, w.astype(np.float64).sum(axis=1), "row sums")
+
+
+def test_group_split_norm_argument_errors(dev):
+    w, x, d = dev.upload(_wx(9, 64, 16)), dev.upload(np.ones(64, np.float32)), dev.alloc(64)
+    base = {"vx": w, "y": x, "dst": d, "ncols": 64, "nrows": 16}
+    for bad in ({"dst_scaled": d}, {"scale_weight": x}, {"sumsq_out": d, "norm_weight": x},
+                {"sumsq_out": d, "vx_up": w}, {"sumsq_in": x, "norm_weight": x, "norm_eps": 1e-5},
+                {"dst_scaled": d, "scale_weight": x, "sumsq_in": x}):
+        with pytest.raises(GaloisHipError):
+            dev.dequantize_mul_mat_vec_q4_0_group([dict(base, **bad)])
+    with pytest.raises(GaloisHipError):   # modes may not be mixed in one call
+        dev.dequantize_mul_mat_vec_q4_0_group([dict(base, sumsq_in=x, norm_eps=1e-5), dict(base)])
+    for t in (w, x, d):
+        dev.free(t)
 
 
 def test_group_argument_errors(dev):

@@ -91,7 +91,7 @@ def test_decode_step_matches_oracle_with_a_filled_cache(gdev):
     dec = g.LlamaDecoder(gdev, **hp)
     _load(dec, w, kc, vc)
     ref = _ref_step(w, hp, kc.copy(), vc.copy(), 123, n_past)
-    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1), (3, 5, 1)):
+    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1), (3, 5, 1), (4, 5, 1)):
         _load(dec, w, kc, vc)
         dec.decode(123, n_past, fused)
         _check(dec.logits(), ref, 1e-4)
@@ -121,7 +121,7 @@ def test_decode_from_an_empty_cache_over_several_tokens(gdev):
     vc = np.zeros_like(kc)
     for n_past, tok in enumerate([1, 400, 17, 17, 511]):
         ref = _ref_step(w, hp, kc, vc, tok, n_past)
-        dec.decode(tok, n_past, (0, 3, 2, 1, 3)[n_past])   # every launch plan in turn, on one cache
+        dec.decode(tok, n_past, (0, 3, 2, 4, 1)[n_past])   # every launch plan in turn, on one cache
         _check(dec.logits(), ref, 1e-4)
     dec.close()
 
