@@ -87,6 +87,30 @@ __device__ __forceinline__ void at_combine(const float *rec, float *__restrict__
                                            float (*red)[AT_THREADS / 64]) {
     constexpr int WAVES = AT_THREADS / 64;
     const int d = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (S <= 16) {
+        // Few splits (up to 2048 keys): every thread fetches all maxima, sums and its own element of every partial
+        // output in one go -- one trip to memory instead of three dependent ones, and no barrier.  Same order of
+        // additions as the general path below.
+        float ms[16], ss[16], os[16];
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            const float *r = rec + (size_t)min(s, S - 1) * (D + 4);
+            ms[s] = at_load(r), ss[s] = at_load(r + 1), os[s] = at_load(r + 4 + min(d, D - 1));
+        }
+        float M = ms[0];
+#pragma unroll
+        for (int s = 1; s < 16; s++) M = fmaxf(M, s < S ? ms[s] : M);
+        float den = 0.0f, num = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 16; s++)
+            if (s < S) {
+                const float ws = expf(ms[s] - M);
+                den = __builtin_fmaf(ws, ss[s], den);
+                num = __builtin_fmaf(ws, os[s], num);
+            }
+        if (d < D) out_h[d] = num / den;
+        return;
+    }
     float mx = -__builtin_inff();
     for (int s = d; s < S; s += AT_THREADS) {
         const float ms = at_load(rec + (size_t)s * (D + 4));
