@@ -167,9 +167,9 @@ __device__ __forceinline__ float slot_dot(const q4_slot &q, const uint32_t (&xl)
     const float dA = f16_bits_to_f32(q.w[0] & 0xFFFFu);
     const float dB = f16_bits_to_f32(q.w[4] >> 16);
     const uint32_t sign = 0x88888888u;
-    // block A: qs bytes 0,1 sit in the top half of w[0], bytes 14,15 in the low half of w[4]
-    const uint32_t ndA[4] = {__builtin_amdgcn_alignbit(q.w[4], q.w[0], 16) ^ sign, q.w[1] ^ sign, q.w[2] ^ sign,
-                             q.w[3] ^ sign};
+    // block A's qs start 2 bytes into the slot: each of its dwords is the top half of one word and the low half of the next
+    const uint32_t ndA[4] = {__builtin_amdgcn_alignbit(q.w[1], q.w[0], 16) ^ sign, __builtin_amdgcn_alignbit(q.w[2], q.w[1], 16) ^ sign,
+                             __builtin_amdgcn_alignbit(q.w[3], q.w[2], 16) ^ sign, __builtin_amdgcn_alignbit(q.w[4], q.w[3], 16) ^ sign};
     const uint32_t ndB[4] = {q.w[5] ^ sign, q.w[6] ^ sign, q.w[7] ^ sign, q.w[8] ^ sign};
     const int tA = block_dot<L>(ndA, xl, 0);
     const int tB = block_dot<L>(ndB, xl, 4);

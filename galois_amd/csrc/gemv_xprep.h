@@ -41,15 +41,12 @@ GH_HD float bits_f32(uint32_t u) {
     return f;
 }
 
-// Byte of the 16-byte qs array that nibble pair t (0..3) of weight-dword group g (0..7) holds.
-// A 36-byte slot is two blocks: block A's qs start 2 bytes into the slot, so its bytes
-// 0,1 and 14,15 share dwords with the two f16 scales and are gathered into group 0
-// ("edge"); groups 1..3 are bytes 2-5, 6-9, 10-13; block B's groups 4..7 are aligned.
-GH_HD int group_byte(int g, int t) {
-    if (g >= 4) return 4 * (g - 4) + t;
-    if (g == 0) return t < 2 ? t : 12 + t;
-    return 4 * g - 2 + t;
-}
+// Byte of the 16-byte qs array that nibble pair t (0..3) of weight-dword group g (0..7) holds:
+// groups 0..3 are bytes 0-3, 4-7, 8-11, 12-15 of block A, groups 4..7 the same of block B.
+// (A 36-byte slot is two blocks; block A's qs start 2 bytes into the slot, so the kernel
+// assembles each of its four dwords from two neighbouring ones.)  A group's activations are
+// then two runs of four consecutive floats, 16 apart: two aligned 16-byte pieces.
+GH_HD int group_byte(int g, int t) { return 4 * (g & 3) + t; }
 
 // Index (within the 64 activations of a slot) of nibble j (0..7) of group g:
 // even nibbles are the low nibbles (weight b), odd nibbles the high nibbles (weight 16+b).
