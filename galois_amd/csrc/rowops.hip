@@ -42,14 +42,21 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_rows(const float *__res
     __shared__ float part[kNormThreads / 64];
     const size_t base = (size_t)blockIdx.x * ncols;
     const int nvec = ncols >> 2;
-    float4 v[NV];
+    float4 v[NV], g[NV];
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         const int c = threadIdx.x + i * kNormThreads;
         v[i] = c < nvec ? reinterpret_cast<const float4 *>(x + base)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
     }
+    // the weight is requested behind the row, before the reduction, so that nothing waits for it afterwards
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = threadIdx.x + i * kNormThreads;
+        g[i] = (w && c < nvec) ? reinterpret_cast<const float4 *>(w)[c] : make_float4(1.f, 1.f, 1.f, 1.f);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
@@ -62,10 +69,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_rows(const float *__res
         const int c = threadIdx.x + i * kNormThreads;
         if (c < nvec) {
             float4 o = make_float4(v[i].x * scale, v[i].y * scale, v[i].z * scale, v[i].w * scale);
-            if (w) {
-                const float4 g = reinterpret_cast<const float4 *>(w)[c];
-                o.x *= g.x, o.y *= g.y, o.z *= g.z, o.w *= g.w;
-            }
+            if (w) o.x *= g[i].x, o.y *= g[i].y, o.z *= g[i].z, o.w *= g[i].w;
             reinterpret_cast<float4 *>(y + base)[c] = o;
         }
     }
@@ -136,19 +140,29 @@ __global__ __launch_bounds__(kRopeThreads) void rope_rows(const float *__restric
     const int row_hi = min(row_lo + p_delta_rows, nrows);
     const float p0 = (float)pos[group] * freq_scale;
     for (int pi = lane; pi < npairs; pi += 64) {
+        int r = row_lo + wave;
+        // RU rows in flight per lane; the first RU are requested before the angle's sine and cosine are computed
+        // (a few hundred instructions), so the arithmetic runs while they are in flight
+        constexpr int RU = 4, RS = kRopeThreads / 64;
+        float2 first[RU];
+        const bool have_first = r + (RU - 1) * RS < row_hi;  // wave-uniform
+        if (have_first) {
+#pragma unroll
+            for (int u = 0; u < RU; u++) first[u] = reinterpret_cast<const float2 *>(x + (size_t)(r + u * RS) * ncols)[pi];
+        }
         const float theta = p0 * powf(theta_scale, (float)pi);
         float sn, cs;
         sincosf(theta, &sn, &cs);
-        int r = row_lo + wave;
-        // four rows in flight per lane
-        for (; r + 3 * (kRopeThreads / 64) < row_hi; r += 4 * (kRopeThreads / 64)) {
-            float2 v[4];
+        bool use_first = have_first;
+        for (; r + (RU - 1) * RS < row_hi; r += RU * RS) {
+            float2 v[RU];
 #pragma unroll
-            for (int u = 0; u < 4; u++)
-                v[u] = reinterpret_cast<const float2 *>(x + (size_t)(r + u * (kRopeThreads / 64)) * ncols)[pi];
+            for (int u = 0; u < RU; u++)
+                v[u] = use_first ? first[u] : reinterpret_cast<const float2 *>(x + (size_t)(r + u * RS) * ncols)[pi];
+            use_first = false;
 #pragma unroll
-            for (int u = 0; u < 4; u++)
-                reinterpret_cast<float2 *>(y + (size_t)(r + u * (kRopeThreads / 64)) * ncols)[pi] =
+            for (int u = 0; u < RU; u++)
+                reinterpret_cast<float2 *>(y + (size_t)(r + u * RS) * ncols)[pi] =
                     make_float2(__builtin_fmaf(v[u].x, cs, -(v[u].y * sn)), __builtin_fmaf(v[u].x, sn, v[u].y * cs));
         }
         for (; r < row_hi; r += kRopeThreads / 64) {
