@@ -37,14 +37,37 @@ __global__ __launch_bounds__(kEwThreads) void ew_scale(const float *__restrict__
     if (i < k) dst[i] = scale * x[i];
 }
 
+// Four elements per thread when k % 4 == 0 and the pointers are 16-byte aligned.
+__global__ __launch_bounds__(kEwThreads) void ew_scale4(const float4 *__restrict__ x, float4 *__restrict__ dst,
+                                                        float scale, int64_t k4) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i >= k4) return;
+    const float4 a = x[i];
+    dst[i] = make_float4(scale * a.x, scale * a.y, scale * a.z, scale * a.w);
+}
+
+__device__ __forceinline__ float silu1(float v) { return v / (1.0f + expf(-v)); }
+
 // silu_f32 (unary.cu:1-10): x / (1 + exp(-x)); with `up` != nullptr the SwiGLU product silu(x) * up.
 __global__ __launch_bounds__(kEwThreads) void ew_silu(const float *__restrict__ x, const float *__restrict__ up,
                                                       float *__restrict__ dst, int64_t k) {
     const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
     if (i >= k) return;
-    const float v = x[i];
-    const float s = v / (1.0f + expf(-v));
+    const float s = silu1(x[i]);
     dst[i] = up ? s * up[i] : s;
+}
+
+__global__ __launch_bounds__(kEwThreads) void ew_silu4(const float4 *__restrict__ x, const float4 *__restrict__ up,
+                                                       float4 *__restrict__ dst, int64_t k4) {
+    const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (i >= k4) return;
+    const float4 v = x[i];
+    float4 s = make_float4(silu1(v.x), silu1(v.y), silu1(v.z), silu1(v.w));
+    if (up) {
+        const float4 u = up[i];
+        s.x *= u.x, s.y *= u.y, s.z *= u.z, s.w *= u.w;
+    }
+    dst[i] = s;
 }
 
 // cpy_f32_f32 / cpy_f32_f16 (cpy.cu:79-156): element i of a [ne00, ne01, *] source with byte
@@ -131,8 +154,12 @@ int32_t galois_hip_scale_f32(galois_hip_ctx *ctx, const float *x, float *dst, fl
     GH_REQUIRE(ctx, k > 0 && k <= (int64_t)0x7FFFFFFF * kEwThreads, GALOIS_HIP_E_SHAPE, "scale_f32");
     GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "scale_f32");
     GH_BIND(ctx);
-    hipLaunchKernelGGL(ew_scale, dim3((unsigned)((k + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0, ctx->stream,
-                       x, dst, scale, k);
+    if (k % 4 == 0 && gh_aligned(x, 16) && gh_aligned(dst, 16))
+        hipLaunchKernelGGL(ew_scale4, dim3((unsigned)((k / 4 + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0,
+                           ctx->stream, (const float4 *)x, (float4 *)dst, scale, k / 4);
+    else
+        hipLaunchKernelGGL(ew_scale, dim3((unsigned)((k + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0,
+                           ctx->stream, x, dst, scale, k);
     GH_LAUNCH_CHECK(ctx, "scale_f32 launch");
 }
 
@@ -143,8 +170,12 @@ static int32_t launch_silu(galois_hip_ctx *ctx, const float *x, const float *up,
     GH_REQUIRE(ctx, k > 0 && k <= (int64_t)0x7FFFFFFF * kEwThreads, GALOIS_HIP_E_SHAPE, what);
     GH_REQUIRE(ctx, gh_aligned(x, 4) && gh_aligned(up, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, what);
     GH_BIND(ctx);
-    hipLaunchKernelGGL(ew_silu, dim3((unsigned)((k + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0, ctx->stream,
-                       x, up, dst, k);
+    if (k % 4 == 0 && gh_aligned(x, 16) && gh_aligned(up, 16) && gh_aligned(dst, 16))
+        hipLaunchKernelGGL(ew_silu4, dim3((unsigned)((k / 4 + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0,
+                           ctx->stream, (const float4 *)x, (const float4 *)up, (float4 *)dst, k / 4);
+    else
+        hipLaunchKernelGGL(ew_silu, dim3((unsigned)((k + kEwThreads - 1) / kEwThreads)), dim3(kEwThreads), 0,
+                           ctx->stream, x, up, dst, k);
     GH_LAUNCH_CHECK(ctx, what);
 }
 

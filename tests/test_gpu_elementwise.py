@@ -26,9 +26,9 @@ def test_add_mul_broadcast(dev, kx, ky):
         dev.free(b)
 
 
-def test_scale_silu(dev):
+@pytest.mark.parametrize("k", [11008, 11007, 3, 4, 1 << 20])   # multiples of 4 take the four-per-thread kernels
+def test_scale_silu(dev, k):
     rng = np.random.default_rng(5)
-    k = 11008
     x, u = (rng.standard_normal(k) * 3).astype(np.float32), rng.standard_normal(k).astype(np.float32)
     xb, ub, ob = dev.upload(x), dev.upload(u), _out(dev, k)
     dev.scale_f32(xb, ob, 0.08838834764831845, k)
