@@ -234,7 +234,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--cpu-seconds", type=float, default=8.0, help="CPU baseline budget per thread setting")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget per thread setting")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip prefill / row-kernel side measurements")
     ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode-step measurement")
