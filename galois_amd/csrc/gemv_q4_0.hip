@@ -19,19 +19,6 @@
 
 #include <type_traits>
 
-// Phase timestamps for tuning builds (-DGEMV_TIMING): one s_memtime per phase per wave.
-#ifdef GEMV_TIMING
-__device__ unsigned long long *g_gemv_tbuf;
-#define GH_TSTAMP(i)                                                                                   \
-    do {                                                                                               \
-        if ((threadIdx.x & 63) == 0)                                                                   \
-            g_gemv_tbuf[((size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + (i)] = \
-                __builtin_amdgcn_s_memtime();                                                          \
-    } while (0)
-#else
-#define GH_TSTAMP(i)
-#endif
-
 namespace {
 
 constexpr int kChunkSlots = 192;  // slots staged per pass over LDS (12288 activations)
@@ -202,7 +189,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
     for (int g = 0; g < G; g++)
 #pragma unroll
         for (int r = 0; r < R; r++) acc[g][r] = 0.0f;
-    GH_TSTAMP(0);
 
     for (int c0 = 0; c0 < (MULTIPASS ? nslots : 1); c0 += kChunkSlots) {
         const int cs = MULTIPASS ? min(kChunkSlots, nslots - c0) : nslots;
@@ -217,11 +203,8 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
             for (int r = 0; r < R; r++)
                 load_slot(q0[r], W + (size_t)min(row0 + r, N - 1) * row_bytes + (size_t)s * sizeof(q4_slot));
         }
-        GH_TSTAMP(1);
         xp.compute(lds, cs);
-        GH_TSTAMP(2);
         __syncthreads();
-        GH_TSTAMP(3);
 
         for (int sl = lane; sl - lane < cs; sl += 64) {  // uniform trip count; lanes past the end idle
             const bool act = sl < cs;
@@ -261,7 +244,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
         }
     }
 
-    GH_TSTAMP(4);
     // every total lands in lane 63; lane 63-j picks up row j so the wave stores its rows at once
     float out = 0.0f;
 #pragma unroll
@@ -273,7 +255,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
             if (lane == g * R + r) out = b;
         }
     if (lane < R * G && row0 + lane < N) y[row0 + lane] = out;
-    GH_TSTAMP(5);
 }
 
 // Generic path: any K % 32 == 0 and any 2-byte-aligned W / 4-byte-aligned x.
@@ -362,7 +343,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     constexpr bool NARG = NORM_MODE != 0;    // the norm_w / eps arguments are used
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    GH_TSTAMP(0);
 
     // Every product's fields are fetched before any is chosen (the empty asm makes each an opaque value; left
     // alone, the compiler turns a select of two arguments into a second, dependent load from a selected address).
@@ -412,7 +392,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     const int wg_row0 = ((int)blockIdx.x - first_blk) * (WAVES * rw * groups);
     int row0 = wg_row0 + wave * rw;
     const size_t row_bytes = (size_t)ns * sizeof(q4_slot);
-    GH_TSTAMP(1);
 
     float acc[R];
 #pragma unroll
@@ -480,7 +459,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                 load_slot(q0[j], base + (size_t)row * row_bytes + (size_t)s * sizeof(q4_slot));
             }
         }
-        GH_TSTAMP(2);
         // Where the results go, fetched now (indexed argument loads) so that nothing waits for them at the end.
         dst_bits = (uint64_t)a.dst[ii], res_bits = (uint64_t)a.residual[ii];
         asm volatile("" : "+s"(dst_bits));
@@ -572,9 +550,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             }
         }
     }
-    GH_TSTAMP(3);
     __syncthreads();
-    GH_TSTAMP(4);
     float inv2 = 1.0f;
     if (NORM2) {
         float tot = 0.0f;
@@ -678,7 +654,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             ((float *)(global_out)ssq_bits)[(int)blockIdx.x - first_blk] = tot;
         }
     }
-    GH_TSTAMP(6);
 }
 
 template <int L, int R, int G, int WAVES, int OCC>
