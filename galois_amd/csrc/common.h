@@ -11,9 +11,6 @@ struct galois_hip_ctx {
     int32_t ordinal;
     hipStream_t stream;
     int32_t n_cu;
-    int32_t gemv_config;  // 0 = choose from the shape; GALOIS_HIP_GEMV_CONFIG=1..6 forces a kernel shape (tuning)
-    int32_t gemm_tile_n;  // 0 = choose from the shape; GALOIS_HIP_GEMM_TILE_N=48|96 forces the prefill tile width (tuning)
-    int32_t gemv_units_per_wave;  // 0 = choose from the shape; GALOIS_HIP_GEMV_UNITS forces it (tuning)
     void *ws;         // workspace owned by the context (fp16 activations of the prefill matmul)
     size_t ws_bytes;
     void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul, partial results of the decode attention

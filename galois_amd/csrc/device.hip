@@ -2,7 +2,6 @@
 // obtains from cudarc).  One context = one device ordinal + one stream.
 #include "common.h"
 
-#include <stdlib.h>
 
 extern "C" {
 
@@ -41,12 +40,6 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     ctx->scratch = nullptr;
     ctx->attn_done = nullptr;
     ctx->capturing = false;
-    const char *cfg = getenv("GALOIS_HIP_GEMV_CONFIG");
-    ctx->gemv_config = cfg ? atoi(cfg) : 0;
-    const char *gtn = getenv("GALOIS_HIP_GEMM_TILE_N");
-    ctx->gemm_tile_n = gtn ? atoi(gtn) : 0;
-    const char *upw = getenv("GALOIS_HIP_GEMV_UNITS");
-    ctx->gemv_units_per_wave = upw ? atoi(upw) : 0;
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         delete ctx;

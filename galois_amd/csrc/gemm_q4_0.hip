@@ -578,7 +578,6 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
         const int64_t cus = ctx->n_cu > 0 ? ctx->n_cu : 256;
         const double cost96 = (double)((wg96 + cus - 1) / cus), cost48 = 0.65 * (double)((wg48 + cus - 1) / cus);
         int tile_n = cost48 < cost96 ? 48 : 96;
-        if (ctx->gemm_tile_n == 48 || ctx->gemm_tile_n == 96) tile_n = ctx->gemm_tile_n;
         const int32_t st = tile_n == 48 ? gemm_launch<48>(ctx, (const uint8_t *)W, Xh, Y, K, N, M)
                                         : gemm_launch<96>(ctx, (const uint8_t *)W, Xh, Y, K, N, M);
         if (st != GALOIS_HIP_OK) return st;

@@ -17,8 +17,6 @@
 #include "common.h"
 #include "gemv_xprep.h"
 
-#include <type_traits>
-
 namespace {
 
 constexpr int kChunkSlots = 192;  // slots staged per pass over LDS (12288 activations)
@@ -53,10 +51,14 @@ __device__ __forceinline__ void load_slot(q4_slot &q, const uint8_t *p) {
     for (int i = 0; i < 9; i++) q.w[i] = s[i];  // plain loads: the three loads of a lane share cache lines
 }
 
-// LDS image of one prepared slot: L planes x 8 dwords, then the two block scales.
+// LDS image of one prepared slot: L planes x 8 dwords, then the two block scales and the two scales of the
+// blocks' corrections (0 = the block has none).  The correction planes (gemv_xprep.h) of all slots follow the
+// slots: corr_dwords per slot.
 template <int L>
 struct slot_lds {
     static constexpr int dwords = 8 * L + 4;  // stride = 4 (mod 8): 16-byte reads of 8 lanes hit 32 distinct banks
+    static constexpr int corr_dwords = 8 * xprep::CORR_L;
+    static constexpr int bytes_per_slot = (dwords + corr_dwords) * 4;  // what a launch reserves per slot
 };
 
 // Sum over the 64 lanes of a wave with DPP only; the total lands in lane 63.
@@ -68,6 +70,91 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));  // row_bcast:15
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));  // row_bcast:31
     return v;
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t quad_max(uint32_t v) {
+    return max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true));
+}
+
+// Eight activations of one (slot, weight-dword group) task, in the nibble order of their weight dword, to LDS:
+// the L planes, the block's scale, and -- when the fixed point leaves too much of the block behind -- the
+// correction planes of the residuals with their scale.  The four threads of a quad hold one block.
+template <int L>
+__device__ __forceinline__ void prep_store(float (&x8)[8], uint32_t *slot_dst, uint32_t *corr_dst, int g) {
+    static_assert(L + xprep::CORR_L >= 8, "the task's own LDS words park its eight activations");
+    // max of |x| on the bit patterns: for non-negative floats the unsigned order is the numeric
+    // order, with inf and NaN on top, so a non-finite activation is never lost
+    uint32_t amax = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
+    amax = quad_max<0xB1>(amax);  // quad_perm(1,0,3,2)
+    amax = quad_max<0x4E>(amax);  // quad_perm(2,3,0,1)
+    float mult, scale;
+    xprep::block_scales<L>(amax, &mult, &scale);
+    // What the rounding will leave behind, for the activations below the top binade (the top binade keeps its
+    // 2^-18 relative; in a block without a grid of its own every activation counts as below).
+    const bool no_grid = mult == 0.0f;
+    float sum_r = 0.0f, sum_x = 0.0f;
+    uint32_t rmax = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t xb = __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu;
+        const bool low = no_grid || xprep::below_top_binade(xb, amax);
+        const uint32_t rb = low ? __builtin_bit_cast(uint32_t, xprep::residual(x8[j], mult, scale)) & 0x7FFFFFFFu : 0u;
+        sum_r += __builtin_bit_cast(float, rb);
+        sum_x += low ? __builtin_bit_cast(float, xb) : 0.0f;
+        rmax = max(rmax, rb);
+    }
+    sum_r += dpp_mov<0xB1>(sum_r), sum_x += dpp_mov<0xB1>(sum_x), rmax = quad_max<0xB1>(rmax);
+    sum_r += dpp_mov<0x4E>(sum_r), sum_x += dpp_mov<0x4E>(sum_x), rmax = quad_max<0x4E>(rmax);
+    float scale2 = 0.0f;
+    if (xprep::needs_correction(sum_r, sum_x)) {  // the same in the four threads of the block; rare
+        // The correction planes come first, from the residuals worked out in place of the activations, which wait
+        // in the LDS words this task is about to fill anyway: the rare path must not cost the common one registers.
+        float mult2;
+        xprep::block_scales<xprep::CORR_L>(rmax, &mult2, &scale2);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t *park = j < L ? slot_dst + j * 8 + g : corr_dst + (j - L) * 8 + g;
+            *(volatile uint32_t *)park = __builtin_bit_cast(uint32_t, x8[j]);
+            const uint32_t xb = __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu;
+            x8[j] = (no_grid || xprep::below_top_binade(xb, amax)) ? xprep::residual(x8[j], mult, scale) : 0.0f;
+        }
+        uint32_t planes2[xprep::CORR_L];
+        xprep::make_planes<xprep::CORR_L>(x8, mult2, planes2);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t *park = j < L ? slot_dst + j * 8 + g : corr_dst + (j - L) * 8 + g;
+            x8[j] = __builtin_bit_cast(float, *(const volatile uint32_t *)park);
+        }
+#pragma unroll
+        for (int l = 0; l < xprep::CORR_L; l++) *(volatile uint32_t *)(corr_dst + l * 8 + g) = planes2[l];
+    }
+    uint32_t planes[L];
+    xprep::make_planes<L>(x8, mult, planes);
+#pragma unroll
+    for (int l = 0; l < L; l++) slot_dst[l * 8 + g] = planes[l];
+    if ((g & 3) == 0) {
+        slot_dst[8 * L + (g >> 2)] = __builtin_bit_cast(uint32_t, scale);
+        slot_dst[8 * L + 2 + (g >> 2)] = __builtin_bit_cast(uint32_t, scale2);
+    }
+}
+
+// What a lane reads of its slot before the dot products.
+template <int L>
+__device__ __forceinline__ uint32_t read_slot_planes(const uint32_t *src, uint32_t (&xl)[L][8], float &sA, float &sB) {
+#pragma unroll
+    for (int l = 0; l < L; l++) {
+        const uint4 a = *reinterpret_cast<const uint4 *>(src + l * 8);
+        const uint4 b = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
+        xl[l][0] = a.x, xl[l][1] = a.y, xl[l][2] = a.z, xl[l][3] = a.w;
+        xl[l][4] = b.x, xl[l][5] = b.y, xl[l][6] = b.z, xl[l][7] = b.w;
+    }
+    const uint4 sc = *reinterpret_cast<const uint4 *>(src + 8 * L);
+    sA = __builtin_bit_cast(float, sc.x);
+    sB = __builtin_bit_cast(float, sc.y);
+    return sc.z | sc.w;  // non-zero: a block of the slot has a correction
 }
 
 // Activation preparation, split in two so that the activation loads can be issued before
@@ -97,29 +184,16 @@ struct xprep_state {
     }
 
     __device__ __forceinline__ void compute(uint32_t *lds, int cs) const {
+        uint32_t *corr = lds + cs * slot_lds<L>::dwords;
 #pragma unroll
         for (int p = 0; p < PG; p++) {
             const int idx = threadIdx.x + p * THREADS;
             if (idx < cs * 8) {
                 const int slot = idx >> 3, g = idx & 7;
                 // nibble order of the weight dword: byte b low, byte b high, byte b+1 low, byte b+1 high, ...
-                const float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
-                                     v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
-                // max of |x| on the bit patterns: for non-negative floats the unsigned order is the numeric
-                // order, with inf and NaN on top, so a non-finite activation is never lost
-                uint32_t amax = 0;
-#pragma unroll
-                for (int j = 0; j < 8; j++) amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
-                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0xB1, 0xF, 0xF, true));
-                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0x4E, 0xF, 0xF, true));
-                float mult, scale;
-                xprep::block_scales<L>(amax, &mult, &scale);
-                uint32_t planes[L];
-                xprep::make_planes<L>(x8, mult, planes);
-                uint32_t *dst = lds + slot * slot_lds<L>::dwords;
-#pragma unroll
-                for (int l = 0; l < L; l++) dst[l * 8 + g] = planes[l];
-                if ((g & 3) == 0) dst[8 * L + (g >> 2)] = __builtin_bit_cast(uint32_t, scale);
+                float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
+                               v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
+                prep_store<L>(x8, lds + slot * slot_lds<L>::dwords, corr + slot * slot_lds<L>::corr_dwords, g);
             }
         }
     }
@@ -165,6 +239,26 @@ __device__ __forceinline__ float slot_dot(const q4_slot &q, const uint32_t (&xl)
     return r;
 }
 
+// The correction of one slot for one row: the slot's weights once more (they are in the caches: the row was just
+// read) against the correction planes of the slot's residuals.
+template <int L>
+__device__ __forceinline__ float slot_correction(const uint8_t *w_slot, const uint32_t *slot_src, const uint32_t *corr_src) {
+    constexpr int CL = xprep::CORR_L;
+    uint32_t xc[CL][8];
+#pragma unroll
+    for (int l = 0; l < CL; l++) {
+        const uint4 a = *reinterpret_cast<const uint4 *>(corr_src + l * 8);
+        const uint4 b = *reinterpret_cast<const uint4 *>(corr_src + l * 8 + 4);
+        xc[l][0] = a.x, xc[l][1] = a.y, xc[l][2] = a.z, xc[l][3] = a.w;
+        xc[l][4] = b.x, xc[l][5] = b.y, xc[l][6] = b.z, xc[l][7] = b.w;
+    }
+    const uint2 sc = *reinterpret_cast<const uint2 *>(slot_src + 8 * L + 2);
+    // a block without a correction has scale 0 and planes nobody wrote: whatever integer they give is multiplied by 0
+    q4_slot q;
+    load_slot(q, w_slot);
+    return slot_dot<CL>(q, xc, __builtin_bit_cast(float, sc.x), __builtin_bit_cast(float, sc.y));
+}
+
 // Fast path: K % 64 == 0, W 4-byte aligned, x 8-byte aligned.
 // Each wave owns R*G consecutive rows; a workgroup owns WAVES*R*G rows.  No explicit
 // register double-buffering: several workgroups share a CU and overlap each other's
@@ -206,24 +300,15 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
         xp.compute(lds, cs);
         __syncthreads();
 
-        for (int sl = lane; sl - lane < cs; sl += 64) {  // uniform trip count; lanes past the end idle
+        uint32_t cmask = 0;  // bit i: this lane's slot of step i has a correction
+        int step = 0;
+        for (int sl = lane; sl - lane < cs; sl += 64, step++) {  // uniform trip count; lanes past the end idle
             const bool act = sl < cs;
             const int s_ld = min(sl, cs - 1);
             uint32_t xl[L][8];
             float sA, sB;
-            {
-                const uint32_t *src = lds + s_ld * SD;
-#pragma unroll
-                for (int l = 0; l < L; l++) {
-                    const uint4 a = *reinterpret_cast<const uint4 *>(src + l * 8);
-                    const uint4 b = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
-                    xl[l][0] = a.x, xl[l][1] = a.y, xl[l][2] = a.z, xl[l][3] = a.w;
-                    xl[l][4] = b.x, xl[l][5] = b.y, xl[l][6] = b.z, xl[l][7] = b.w;
-                }
-                const uint2 sc = *reinterpret_cast<const uint2 *>(src + 8 * L);
-                sA = __builtin_bit_cast(float, sc.x);
-                sB = __builtin_bit_cast(float, sc.y);
-            }
+            const uint32_t has_corr = read_slot_planes<L>(lds + s_ld * SD, xl, sA, sB);
+            if (act && has_corr) cmask |= 1u << step;
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 q4_slot q[R];
@@ -241,6 +326,20 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
                     for (int r = 0; r < R; r++) acc[g][r] += slot_dot<L>(q[r], xl, sA, sB);
                 }
             }
+        }
+        if (cmask) {  // rare: only lanes whose slots have corrections get here
+            const uint32_t *corr = lds + cs * SD;
+            for (int st = 0; st < (kChunkSlots + 63) / 64; st++)
+                if (cmask >> st & 1) {
+                    const int s = st * 64 + lane;
+#pragma unroll
+                    for (int g = 0; g < G; g++)
+#pragma unroll
+                        for (int r = 0; r < R; r++)
+                            acc[g][r] += slot_correction<L>(W + (size_t)min(row0 + g * R + r, N - 1) * row_bytes +
+                                                                (size_t)(c0 + s) * sizeof(q4_slot),
+                                                            lds + s * SD, corr + s * slot_lds<L>::corr_dwords);
+                }
         }
     }
 
@@ -312,7 +411,6 @@ struct gg_args {
     const float *x[GG_MAX];
     int32_t N[GG_MAX];
     int32_t nslots[GG_MAX];
-    int32_t groups[GG_MAX];       // row groups a wave works through, one after the other
     const float *norm_w[GG_MAX];  // NORM 1: RMSNorm weight; NORM 2: the partial sums of squares of the activations
     float *dst[GG_MAX];
     const float *residual[GG_MAX];  // or null
@@ -346,13 +444,13 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
 
     // Every product's fields are fetched before any is chosen (the empty asm makes each an opaque value; left
     // alone, the compiler turns a select of two arguments into a second, dependent load from a selected address).
-    int32_t k_blk0[MAXI], k_N[MAXI], k_ns[MAXI], k_groups[MAXI];
+    int32_t k_blk0[MAXI], k_N[MAXI], k_ns[MAXI];
     uint64_t k_W[MAXI], k_W2[MAXI], k_x[MAXI], k_nw[NARG ? MAXI : 1];  // pointers as bits: an address that has been
                                                 // through an asm is no longer known to be global memory and is cast back below
     float k_eps[NARG ? MAXI : 1];
 #pragma unroll
     for (int k = 0; k < MAXI; k++) {
-        k_blk0[k] = a.blk0[k], k_N[k] = a.N[k], k_ns[k] = a.nslots[k], k_groups[k] = a.groups[k];
+        k_blk0[k] = a.blk0[k], k_N[k] = a.N[k], k_ns[k] = a.nslots[k];
         k_W[k] = (uint64_t)a.W[k], k_W2[k] = (uint64_t)a.W2[k], k_x[k] = (uint64_t)a.x[k];
         if (NARG) k_nw[k] = (uint64_t)a.norm_w[k], k_eps[k] = a.eps[k];
     }
@@ -361,7 +459,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         asm volatile("" : "+s"(k_blk0[k]));
         asm volatile("" : "+s"(k_N[k]));
         asm volatile("" : "+s"(k_ns[k]));
-        asm volatile("" : "+s"(k_groups[k]));
         asm volatile("" : "+s"(k_W[k]));
         asm volatile("" : "+s"(k_W2[k]));
         asm volatile("" : "+s"(k_x[k]));
@@ -373,13 +470,13 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     int ii = 0, first_blk = 0;
     uint64_t W_bits = k_W[0], W2_bits = k_W2[0], x_bits = k_x[0], nw_bits = NARG ? k_nw[0] : 0;
     float eps = NARG ? k_eps[0] : 0.0f;
-    int N = k_N[0], ns = k_ns[0], groups = k_groups[0];
+    int N = k_N[0], ns = k_ns[0];
 #pragma unroll
     for (int k = 1; k < MAXI; k++) {
         const bool ge = (int)blockIdx.x >= k_blk0[k];
         ii = ge ? k : ii, first_blk = ge ? k_blk0[k] : first_blk;
         W_bits = ge ? k_W[k] : W_bits, W2_bits = ge ? k_W2[k] : W2_bits, x_bits = ge ? k_x[k] : x_bits;
-        N = ge ? k_N[k] : N, ns = ge ? k_ns[k] : ns, groups = ge ? k_groups[k] : groups;
+        N = ge ? k_N[k] : N, ns = ge ? k_ns[k] : ns;
         if (NARG) nw_bits = ge ? k_nw[k] : nw_bits, eps = ge ? k_eps[k] : eps;
     }
     typedef const __attribute__((address_space(1))) uint8_t *global_bytes;
@@ -388,9 +485,8 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     const float *const xg = (const float *)(global_floats)x_bits;
     const bool dual = W2 != nullptr;
     const int rw = dual ? R / 2 : R;  // rows per wave and group
-    // group g of the workgroup's waves covers WAVES * rw consecutive rows: neighbouring waves read neighbouring rows
-    const int wg_row0 = ((int)blockIdx.x - first_blk) * (WAVES * rw * groups);
-    int row0 = wg_row0 + wave * rw;
+    // the workgroup's waves cover WAVES * rw consecutive rows: neighbouring waves read neighbouring rows
+    const int row0 = ((int)blockIdx.x - first_blk) * (WAVES * rw) + wave * rw;
     const size_t row_bytes = (size_t)ns * sizeof(q4_slot);
 
     float acc[R];
@@ -402,7 +498,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     // are in flight.
     q4_slot q0[R];
     uint64_t dst_bits, res_bits, dst2_bits = 0, scale2_bits = 0, ssq_bits = 0;
-    float scale2_first = 0.0f;
+    float scale2_first = 0.0f;  // OUT2: scale_weight of this lane's row
     {
         const float *wg = NORM ? (const float *)(global_floats)nw_bits : nullptr;
         float2 v[PG][4], nw[NORM ? PG : 1][4];
@@ -469,10 +565,6 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             asm volatile("" : "+s"(scale2_bits));
             asm volatile("" : "+s"(ssq_bits));
         }
-        if (OUT2) {  // the first group's scale values ride behind the weights (always a load: see the activations)
-            const float *sp = scale2_bits ? (const float *)(global_floats)scale2_bits + min(row0 + (lane < rw ? lane : 0), N - 1) : xg;
-            scale2_first = *sp;
-        }
         if (NORM2) {  // the partial sums reach every wave through the barrier that publishes the planes
             psq = wave_sum(psq);
             if (lane == 0) red[wave] = psq;
@@ -527,30 +619,24 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                     }
             }
         }
+        // the corrections live behind the slots (and behind the staged activations, which other threads may still read)
+        uint32_t *const corr = lds + ns * SD + (STAGED ? ns * 64 : 0);
 #pragma unroll
         for (int p = 0; p < PG; p++) {
             const int idx = threadIdx.x + p * THREADS;
             if (idx < ns * 8) {
                 const int slot = idx >> 3, g = idx & 7;
-                const float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
-                                     v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
-                uint32_t amax = 0;
-#pragma unroll
-                for (int j = 0; j < 8; j++) amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
-                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0xB1, 0xF, 0xF, true));
-                amax = max(amax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)amax, 0x4E, 0xF, 0xF, true));
-                float mult, scale;
-                xprep::block_scales<L>(amax, &mult, &scale);
-                uint32_t planes[L];
-                xprep::make_planes<L>(x8, mult, planes);
-                uint32_t *dst = lds + slot * SD;
-#pragma unroll
-                for (int l = 0; l < L; l++) dst[l * 8 + g] = planes[l];
-                if ((g & 3) == 0) dst[8 * L + (g >> 2)] = __builtin_bit_cast(uint32_t, scale);
+                float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
+                               v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
+                prep_store<L>(x8, lds + slot * SD, corr + slot * slot_lds<L>::corr_dwords, g);
             }
         }
     }
     __syncthreads();
+    if (OUT2) {  // the scale values ride behind the weights, requested once the preparation's registers are free
+        const float *sp = scale2_bits ? (const float *)(global_floats)scale2_bits + min(row0 + (lane < rw ? lane : 0), N - 1) : xg;
+        scale2_first = *sp;
+    }
     float inv2 = 1.0f;
     if (NORM2) {
         float tot = 0.0f;
@@ -561,30 +647,19 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     }
     float sq_out = 0.0f;  // OUT2: squares of this lane's results
 
-    // One group of rows.  The first group's first slots are the ones requested before the preparation; it is
-    // peeled off the loop so that those registers are not kept alive through the later groups.
-    auto do_group = [&](auto first_tag) {
-        constexpr bool FIRST = decltype(first_tag)::value;
-        for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
+    // The rows of this wave.  The first slots are the ones requested before the preparation.
+    {
+        uint32_t cmask = 0;  // bit i: this lane's slot of step i has a correction
+        int step = 0;
+        for (int sl = lane; sl - lane < ns; sl += 64, step++) {  // uniform trip count; lanes past the end idle
             const bool act = sl < ns;
             const int s_ld = min(sl, ns - 1);
             uint32_t xl[L][8];
             float sA, sB;
-            {
-                const uint32_t *src = lds + s_ld * SD;
-#pragma unroll
-                for (int l = 0; l < L; l++) {
-                    const uint4 lo4 = *reinterpret_cast<const uint4 *>(src + l * 8);
-                    const uint4 hi4 = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
-                    xl[l][0] = lo4.x, xl[l][1] = lo4.y, xl[l][2] = lo4.z, xl[l][3] = lo4.w;
-                    xl[l][4] = hi4.x, xl[l][5] = hi4.y, xl[l][6] = hi4.z, xl[l][7] = hi4.w;
-                }
-                const uint2 sc = *reinterpret_cast<const uint2 *>(src + 8 * L);
-                sA = __builtin_bit_cast(float, sc.x);
-                sB = __builtin_bit_cast(float, sc.y);
-            }
+            const uint32_t has_corr = read_slot_planes<L>(lds + s_ld * SD, xl, sA, sB);
+            if (act && has_corr) cmask |= 1u << step;
             q4_slot q[R];
-            if (FIRST && sl == lane) {
+            if (sl == lane) {
 #pragma unroll
                 for (int j = 0; j < R; j++) q[j] = q0[j];
             } else {
@@ -599,6 +674,20 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
 #pragma unroll
                 for (int j = 0; j < R; j++) acc[j] += slot_dot<L>(q[j], xl, sA, sB);
             }
+        }
+        if (cmask) {  // rare: only lanes whose slots have corrections get here
+            const uint32_t *corr = lds + ns * SD + ((NORM && PG == 1) ? ns * 64 : 0);
+            for (int st = 0; st < (GG_MAX_SLOTS + 63) / 64; st++)
+                if (cmask >> st & 1) {
+                    const int s = st * 64 + lane;
+#pragma unroll
+                    for (int j = 0; j < R; j++) {
+                        const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
+                        const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
+                        acc[j] += slot_correction<L>(base + (size_t)row * row_bytes + (size_t)s * sizeof(q4_slot),
+                                                     lds + s * SD, corr + s * slot_lds<L>::corr_dwords);
+                    }
+                }
         }
 
         // every total lands in lane 63; lane j picks up row j so the wave stores its rows at once
@@ -628,19 +717,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             ((float *)(global_out)dst_bits)[row0 + lane] = out;
             if (OUT2) {
                 if (dst2_bits)
-                    ((float *)(global_out)dst2_bits)[row0 + lane] =
-                        out * (FIRST ? scale2_first : ((const float *)(global_floats)scale2_bits)[row0 + lane]);
+                    ((float *)(global_out)dst2_bits)[row0 + lane] = out * scale2_first;
                 sq_out = __builtin_fmaf(out, out, sq_out);
             }
         }
-#pragma unroll
-        for (int j = 0; j < R; j++) acc[j] = 0.0f;
-    };
-    do_group(std::true_type{});
-    for (int g = 1; g < groups; g++) {
-        row0 += WAVES * rw;
-        if (row0 >= N) break;  // wave-uniform
-        do_group(std::false_type{});
     }
     if (OUT2 && ssq_bits) {  // wave-uniform; every wave of the workgroup gets here
         sq_out = wave_sum(sq_out);
@@ -661,7 +741,7 @@ void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst
     const int rows_per_wg = WAVES * R * G;
     const dim3 grid((N + rows_per_wg - 1) / rows_per_wg), block(WAVES * 64);
     const int pass_slots = min(nslots, kChunkSlots);
-    const size_t lds = (size_t)pass_slots * slot_lds<L>::dwords * sizeof(uint32_t);
+    const size_t lds = (size_t)pass_slots * slot_lds<L>::bytes_per_slot;
     constexpr int PGMAX = (kChunkSlots * 8 + WAVES * 64 - 1) / (WAVES * 64);
     constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
     const uint8_t *W = (const uint8_t *)vx;
@@ -672,8 +752,8 @@ void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst
         hipLaunchKernelGGL((gemv_q4_0_dot8<L, R, G, WAVES, PGMAX, OCC, false>), grid, block, lds, ctx->stream, W, x,
                            dst, nslots, N);
     else
-        hipLaunchKernelGGL((gemv_q4_0_dot8<L, R, G, WAVES, PGMAX, OCC, true>), grid, block, lds, ctx->stream, W, x,
-                           dst, nslots, N);
+        hipLaunchKernelGGL((gemv_q4_0_dot8<L, R, G, WAVES, PGMAX, (OCC > 3 ? 3 : OCC), true>), grid, block, lds,
+                           ctx->stream, W, x, dst, nslots, N);  // the loop over passes keeps more alive
 }
 
 // Host side of the group kernel: checks, the block range of every matrix, launch.
@@ -682,10 +762,10 @@ void launch_dot8(galois_hip_ctx *ctx, const void *vx, const float *x, float *dst
 template <int L, int R, int WAVES, int OCC, int MAXI>
 void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, int max_slots, int mode, bool out2) {
     const dim3 grid(blocks), block(WAVES * 64);
-    const size_t lds = (size_t)max_slots * slot_lds<L>::dwords * sizeof(uint32_t);
+    const size_t lds = (size_t)max_slots * slot_lds<L>::bytes_per_slot;
     constexpr int PGMAX = (kChunkSlots * 8 + WAVES * 64 - 1) / (WAVES * 64);
     constexpr int PGSMALL = (64 * 8 + WAVES * 64 - 1) / (WAVES * 64);  // K <= 4096
-    constexpr int OCCN = OCC > 4 ? 4 : OCC;  // the normalising preparation of a long vector needs more than 64 registers
+    constexpr int OCCN = OCC > 4 ? 4 : OCC;  // the normalising preparation of a long vector needs more registers
 #define GG_LAUNCH(PG_, OCC_, MODE_, OUT2_, LDS_) \
     hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PG_, OCC_, MODE_, MAXI, OUT2_>), grid, block, LDS_, ctx->stream, a)
     if (max_slots <= 64) {
@@ -747,7 +827,7 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
         GH_REQUIRE(ctx, (s.dst_scaled == nullptr) == (s.scale_weight == nullptr), GALOIS_HIP_E_NULL,
                    "gemv group: dst_scaled and scale_weight go together");
         if (s.dst_scaled || s.sumsq_out) {
-            GH_REQUIRE(ctx, m == 0 && !s.vx_up && n_items <= 4 && ctx->gemv_units_per_wave <= 1, GALOIS_HIP_E_UNSUPPORTED,
+            GH_REQUIRE(ctx, m == 0 && !s.vx_up && n_items <= 4, GALOIS_HIP_E_UNSUPPORTED,
                        "gemv group: dst_scaled / sumsq_out are written by plain products (no norm, no pair) in calls of at most four");
             GH_REQUIRE(ctx, gh_aligned(s.dst_scaled, 4) && gh_aligned(s.scale_weight, 4) && gh_aligned(s.sumsq_out, 4),
                        GALOIS_HIP_E_ALIGN, "gemv group: 4-byte aligned vectors");
@@ -763,30 +843,23 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     }
     // Workgroup shape by rows per CU, as for the one-product kernel: few rows -> 16 waves x 1 slot so every SIMD has
     // work; more rows -> 8 waves x 2 slots, three workgroups resident per CU.  A gate / up pair needs 2 slots per lane.
+    // One 16-slot row group per workgroup: measured, working through two or four groups per workgroup (which would
+    // amortise the activation preparation) loses more to the coarser split of the launch than it saves at every
+    // LLaMA-7B shape.
     bool any_dual = false;
     for (int i = 0; i < n_items; i++) any_dual |= items[i].vx_up != nullptr;
-    int cfg = ctx->gemv_config;
-    if (cfg != 1 && cfg != 4 && cfg != 7) cfg = (!any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16) ? 1 : 4;
-    if (any_dual && cfg == 1) cfg = 4;
+    const bool small = !any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16;
     const int slots_per_wg = 16;  // WAVES * R of both shapes
-    // One row group per wave: measured, working through two or four groups per wave (which would amortise the
-    // activation preparation) loses more to the coarser split of the launch than it saves at every LLaMA-7B shape.
     int64_t blocks = 0;
     for (int i = 0; i < n_items; i++) {
-        int groups = ctx->gemv_units_per_wave;
-        if (groups <= 0) groups = 1;
-        groups = groups < 1 ? 1 : (groups > 4 ? 4 : groups);
-        a.groups[i] = groups;
-        const int64_t rows_per_wg = (items[i].vx_up ? slots_per_wg / 2 : slots_per_wg) * groups;
+        const int64_t rows_per_wg = items[i].vx_up ? slots_per_wg / 2 : slots_per_wg;
         a.blk0[i] = (int32_t)blocks;
         blocks += (items[i].nrows + rows_per_wg - 1) / rows_per_wg;
         GH_REQUIRE(ctx, blocks < 0x7FFFFFFF, GALOIS_HIP_E_SHAPE, "gemv group: too many rows");
     }
     GH_BIND(ctx);
-    if (cfg == 1)
+    if (small)
         launch_group_cfg<5, 1, 16, 4>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
-    else if (cfg == 7)
-        launch_group_cfg<5, 2, 8, 8>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
     else
         launch_group_cfg<5, 2, 8, 6>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
     GH_LAUNCH_CHECK(ctx, what);
@@ -809,25 +882,11 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, c
         // Workgroup shape by rows per CU: few rows -> 16 waves x 1 row so every SIMD has work and the
         // activation preparation is spread over 1024 threads; more rows -> 8 waves x 2 rows, several
         // workgroups resident per CU so one's preparation overlaps another's streaming.
-        int cfg = ctx->gemv_config;
-        if (cfg == 6 && ncols <= 64 * GG_MAX_SLOTS) {
-            galois_hip_gemv_item it;
-            memset(&it, 0, sizeof(it));
-            it.vx = vx, it.y = y, it.dst = dst, it.ncols = ncols, it.nrows = nrows;
-            return launch_group(ctx, &it, 1, "dequantize_mul_mat_vec_q4_0");
-        }
-        if (cfg == 0) {
-            const int64_t rows_per_cu = ((int64_t)nrows + ctx->n_cu - 1) / ctx->n_cu;
-            cfg = rows_per_cu <= 16 ? 1 : 4;
-        }
-        switch (cfg) {
-            case 1: launch_dot8<5, 1, 1, 16, 4>(ctx, vx, y, dst, nslots, nrows); break;  // 16 rows per workgroup
-            case 2: launch_dot8<5, 4, 1, 4, 2>(ctx, vx, y, dst, nslots, nrows); break;   // 16 rows, 4 waves
-            case 3: launch_dot8<5, 4, 1, 8, 3>(ctx, vx, y, dst, nslots, nrows); break;   // 32 rows per workgroup
-            case 4: launch_dot8<5, 2, 1, 8, 4>(ctx, vx, y, dst, nslots, nrows); break;   // 16 rows, 8 waves
-            case 5: launch_dot8<6, 4, 1, 4, 2>(ctx, vx, y, dst, nslots, nrows); break;   // 6 activation limbs
-            default: return gh_fail(ctx, GALOIS_HIP_E_UNSUPPORTED, "GALOIS_HIP_GEMV_CONFIG value");
-        }
+        const int64_t rows_per_cu = ((int64_t)nrows + ctx->n_cu - 1) / ctx->n_cu;
+        if (rows_per_cu <= 16)
+            launch_dot8<5, 1, 1, 16, 4>(ctx, vx, y, dst, nslots, nrows);  // 16 rows per workgroup, 16 waves
+        else
+            launch_dot8<5, 2, 1, 8, 4>(ctx, vx, y, dst, nslots, nrows);   // 16 rows per workgroup, 8 waves
     } else {
         hipLaunchKernelGGL(gemv_q4_0_generic, dim3((nrows + 3) / 4), dim3(256), 0, ctx->stream, (const uint16_t *)vx,
                            y, dst, ncols / 32, nrows);

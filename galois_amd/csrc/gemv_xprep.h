@@ -10,6 +10,14 @@
 // holds exactly in integer arithmetic; the only rounding is that of x to XBITS-1 fractional
 // bits below its block's leading power of two (2^-21 relative for 6 limbs).
 //
+// What the rounding drops is not lost.  The residual r = x - X * 2^(e-XBITS+1) is exact in f32.  Activations in
+// the block's top binade (|x| >= 2^e) keep XBITS-1 bits, |r| <= 2^(1-XBITS) |x|; the others share what the common
+// scale leaves them.  A block in which the residuals of those others add up to more than 2^-15 of their sum of |x|
+// (one in which a few activations tower over the rest, so that the rest keeps few bits, or none) gets a correction
+// block: the residuals of those others in the same fixed-point form with their own scale and CORR_L limbs.  The
+// kernel adds dot(weights, correction planes) for such blocks, which takes them to 2^-13 of the largest residual
+// (at most 2^-31 of the block's largest activation); in every other block  sum_{k below the top binade} |r_k| <= 2^-15 * sum_{k below the top binade} |x_k|.
+//
 // Plain C++ (no HIP builtins) so the same code is unit-tested on the CPU.
 #pragma once
 #include <stdint.h>
@@ -78,6 +86,25 @@ GH_HD uint32_t signed_digits(float x, float mult) {
     const uint32_t y = f32_bits(f) - 0x4B400000u + limb_cfg<L>::bias;
     return y ^ limb_cfg<L>::bias;
 }
+
+// What signed_digits rounds away: x - X * scale with X = rne(x * mult) and scale = 1 / mult, exact in f32 (X * scale
+// is a multiple of scale no further than scale / 2 from x, so the difference needs no more bits than x has).
+// A block without a grid (mult = scale = 0: nothing above 2^-100) keeps all of x; a non-finite block gives NaN.
+GH_HD float residual(float x, float mult, float scale) {
+    const float X = __builtin_fmaf(x, mult, 12582912.0f) - 12582912.0f;
+    return __builtin_fmaf(-X, scale, x);
+}
+
+constexpr int CORR_L = 4;                              // limbs of a correction block
+constexpr float CORR_THRESHOLD = 3.0517578125e-05f;    // 2^-15
+
+// Whether |x| (as f32 bits with the sign cleared) lies below the top binade of a block whose largest |x| has the
+// bits amax_bits: only such activations count in the decision below.
+GH_HD bool below_top_binade(uint32_t abs_bits, uint32_t amax_bits) { return abs_bits < (amax_bits & 0x7F800000u); }
+
+// Whether a block gets a correction block, from its sums of |r| and |x| over the activations below the top binade
+// (false for a block with a NaN in it: its scale already poisons the result).
+GH_HD bool needs_correction(float sum_abs_r, float sum_abs_x) { return sum_abs_r > CORR_THRESHOLD * sum_abs_x; }
 
 // 8x8 nibble transpose: in[j] nibble l  ->  out[l] nibble j.
 GH_HD void transpose_nibbles(const uint32_t in[8], uint32_t out[8]) {
