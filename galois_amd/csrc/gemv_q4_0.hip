@@ -80,66 +80,68 @@ __device__ __forceinline__ uint32_t quad_max(uint32_t v) {
 // Eight activations of one (slot, weight-dword group) task, in the nibble order of their weight dword, to LDS:
 // the L planes, the block's scale, and -- when the fixed point leaves too much of the block behind -- the
 // correction planes of the residuals with their scale.  The four threads of a quad hold one block.
-template <int L>
-__device__ __forceinline__ void prep_store(float (&x8)[8], uint32_t *slot_dst, uint32_t *corr_dst, int g) {
-    static_assert(L + xprep::CORR_L >= 8, "the task's own LDS words park its eight activations");
+// refetch(y8) produces the eight activations once more: the rare path takes them from where they came from
+// rather than keep them in registers past the planes, which would cost the common path its occupancy.
+template <int L, class Refetch>
+__device__ __forceinline__ void prep_store(const float (&x8)[8], uint32_t *slot_dst, uint32_t *corr_dst, int g,
+                                           Refetch refetch) {
     // max of |x| on the bit patterns: for non-negative floats the unsigned order is the numeric
     // order, with inf and NaN on top, so a non-finite activation is never lost
     uint32_t amax = 0;
-#pragma unroll
-    for (int j = 0; j < 8; j++) amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
-    amax = quad_max<0xB1>(amax);  // quad_perm(1,0,3,2)
-    amax = quad_max<0x4E>(amax);  // quad_perm(2,3,0,1)
-    float mult, scale;
-    xprep::block_scales<L>(amax, &mult, &scale);
-    // What the rounding will leave behind, for the activations below the top binade (the top binade keeps its
-    // 2^-18 relative; in a block without a grid of its own every activation counts as below).
-    const bool no_grid = mult == 0.0f;
-    float sum_r = 0.0f, sum_x = 0.0f;
-    uint32_t rmax = 0;
+    float sum_x = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const uint32_t xb = __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu;
-        const bool low = no_grid || xprep::below_top_binade(xb, amax);
-        const uint32_t rb = low ? __builtin_bit_cast(uint32_t, xprep::residual(x8[j], mult, scale)) & 0x7FFFFFFFu : 0u;
-        sum_r += __builtin_bit_cast(float, rb);
-        sum_x += low ? __builtin_bit_cast(float, xb) : 0.0f;
-        rmax = max(rmax, rb);
+        amax = max(amax, __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu);
+        sum_x += __builtin_fabsf(x8[j]);
     }
-    sum_r += dpp_mov<0xB1>(sum_r), sum_x += dpp_mov<0xB1>(sum_x), rmax = quad_max<0xB1>(rmax);
-    sum_r += dpp_mov<0x4E>(sum_r), sum_x += dpp_mov<0x4E>(sum_x), rmax = quad_max<0x4E>(rmax);
-    float scale2 = 0.0f;
-    if (xprep::needs_correction(sum_r, sum_x)) {  // the same in the four threads of the block; rare
-        // The correction planes come first, from the residuals worked out in place of the activations, which wait
-        // in the LDS words this task is about to fill anyway: the rare path must not cost the common one registers.
-        float mult2;
-        xprep::block_scales<xprep::CORR_L>(rmax, &mult2, &scale2);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            uint32_t *park = j < L ? slot_dst + j * 8 + g : corr_dst + (j - L) * 8 + g;
-            *(volatile uint32_t *)park = __builtin_bit_cast(uint32_t, x8[j]);
-            const uint32_t xb = __builtin_bit_cast(uint32_t, x8[j]) & 0x7FFFFFFFu;
-            x8[j] = (no_grid || xprep::below_top_binade(xb, amax)) ? xprep::residual(x8[j], mult, scale) : 0.0f;
-        }
-        uint32_t planes2[xprep::CORR_L];
-        xprep::make_planes<xprep::CORR_L>(x8, mult2, planes2);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t *park = j < L ? slot_dst + j * 8 + g : corr_dst + (j - L) * 8 + g;
-            x8[j] = __builtin_bit_cast(float, *(const volatile uint32_t *)park);
-        }
-#pragma unroll
-        for (int l = 0; l < xprep::CORR_L; l++) *(volatile uint32_t *)(corr_dst + l * 8 + g) = planes2[l];
-    }
+    amax = quad_max<0xB1>(amax), sum_x += dpp_mov<0xB1>(sum_x);  // quad_perm(1,0,3,2)
+    amax = quad_max<0x4E>(amax), sum_x += dpp_mov<0x4E>(sum_x);  // quad_perm(2,3,0,1)
+    float mult, scale;
+    xprep::block_scales<L>(amax, &mult, &scale);
     uint32_t planes[L];
     xprep::make_planes<L>(x8, mult, planes);
 #pragma unroll
     for (int l = 0; l < L; l++) slot_dst[l * 8 + g] = planes[l];
+    float scale2 = 0.0f;
+    if (xprep::needs_correction(sum_x, amax, scale)) {  // the same in the four threads of the block; rare
+        const bool no_grid = scale == 0.0f;  // every activation counts as below the top binade
+        float r8[8];
+        refetch(r8);
+        uint32_t rmax = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t xb = __builtin_bit_cast(uint32_t, r8[j]) & 0x7FFFFFFFu;
+            r8[j] = (no_grid || xprep::below_top_binade(xb, amax)) ? xprep::residual(r8[j], mult, scale) : 0.0f;
+            rmax = max(rmax, __builtin_bit_cast(uint32_t, r8[j]) & 0x7FFFFFFFu);
+        }
+        rmax = quad_max<0xB1>(rmax);
+        rmax = quad_max<0x4E>(rmax);
+        float mult2;
+        xprep::block_scales<xprep::CORR_L>(rmax, &mult2, &scale2);
+        uint32_t planes2[xprep::CORR_L];
+        xprep::make_planes<xprep::CORR_L>(r8, mult2, planes2);
+#pragma unroll
+        for (int l = 0; l < xprep::CORR_L; l++) corr_dst[l * 8 + g] = planes2[l];
+    }
     if ((g & 3) == 0) {
         slot_dst[8 * L + (g >> 2)] = __builtin_bit_cast(uint32_t, scale);
         slot_dst[8 * L + 2 + (g >> 2)] = __builtin_bit_cast(uint32_t, scale2);
     }
 }
+
+// The eight activations of task (slot, g) of a vector in global memory, in the order prep_store takes them.
+__device__ __forceinline__ void fetch_task(const float *xs /* the slot's 64 activations */, int g, float2 (&v)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; t += 2) {
+        // nibble pairs t, t+1 of group g: weights (b, b+1) low nibbles and (16+b, 17+b) high nibbles
+        const int b = xprep::group_x_index(g, 2 * t);  // even by construction
+        v[t] = *reinterpret_cast<const float2 *>(xs + b);
+        v[t + 1] = *reinterpret_cast<const float2 *>(xs + b + 16);
+    }
+}
+
+// nibble order of the weight dword: byte b low, byte b high, byte b+1 low, byte b+1 high, ...
+#define GH_TASK_X8(v) {(v)[0].x, (v)[1].x, (v)[0].y, (v)[1].y, (v)[2].x, (v)[3].x, (v)[2].y, (v)[3].y}
 
 // What a lane reads of its slot before the dot products.
 template <int L>
@@ -169,31 +171,26 @@ struct xprep_state {
 #pragma unroll
         for (int p = 0; p < PG; p++) {
             const int idx = threadIdx.x + p * THREADS;
-            if (idx < cs * 8) {
-                const int slot = idx >> 3, g = idx & 7;
-                const float *xs = xg + (size_t)(c0 + slot) * 64;
-#pragma unroll
-                for (int t = 0; t < 4; t += 2) {
-                    // nibble pairs t, t+1 of group g: weights (b, b+1) low nibbles and (16+b, 17+b) high nibbles
-                    const int b = xprep::group_x_index(g, 2 * t);  // even by construction
-                    v[p][t] = *reinterpret_cast<const float2 *>(xs + b);
-                    v[p][t + 1] = *reinterpret_cast<const float2 *>(xs + b + 16);
-                }
-            }
+            if (idx < cs * 8) fetch_task(xg + (size_t)(c0 + (idx >> 3)) * 64, idx & 7, v[p]);
         }
     }
 
-    __device__ __forceinline__ void compute(uint32_t *lds, int cs) const {
+    __device__ __forceinline__ void compute(uint32_t *lds, const float *__restrict__ xg, int c0, int cs) const {
         uint32_t *corr = lds + cs * slot_lds<L>::dwords;
 #pragma unroll
         for (int p = 0; p < PG; p++) {
             const int idx = threadIdx.x + p * THREADS;
             if (idx < cs * 8) {
                 const int slot = idx >> 3, g = idx & 7;
-                // nibble order of the weight dword: byte b low, byte b high, byte b+1 low, byte b+1 high, ...
-                float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
-                               v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
-                prep_store<L>(x8, lds + slot * slot_lds<L>::dwords, corr + slot * slot_lds<L>::corr_dwords, g);
+                const float x8[8] = GH_TASK_X8(v[p]);
+                prep_store<L>(x8, lds + slot * slot_lds<L>::dwords, corr + slot * slot_lds<L>::corr_dwords, g,
+                              [&](float (&y8)[8]) {
+                                  float2 w[4];
+                                  fetch_task(xg + (size_t)(c0 + slot) * 64, g, w);
+                                  const float t8[8] = GH_TASK_X8(w);
+#pragma unroll
+                                  for (int j = 0; j < 8; j++) y8[j] = t8[j];
+                              });
             }
         }
     }
@@ -297,7 +294,9 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
             for (int r = 0; r < R; r++)
                 load_slot(q0[r], W + (size_t)min(row0 + r, N - 1) * row_bytes + (size_t)s * sizeof(q4_slot));
         }
-        xp.compute(lds, cs);
+        // nothing that waits for the activations may be scheduled ahead of the weight requests
+        __builtin_amdgcn_sched_barrier(0);
+        xp.compute(lds, xg, c0, cs);
         __syncthreads();
 
         uint32_t cmask = 0;  // bit i: this lane's slot of step i has a correction
@@ -521,17 +520,8 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
         for (int p = 0; p < PG; p++) {
             const int idx = threadIdx.x + p * THREADS;
             if (!STAGED && idx < ns * 8) {
-                const int slot = idx >> 3, g = idx & 7;
-#pragma unroll
-                for (int t = 0; t < 4; t += 2) {
-                    const int b = slot * 64 + xprep::group_x_index(g, 2 * t);  // even by construction
-                    v[p][t] = *reinterpret_cast<const float2 *>(xg + b);
-                    v[p][t + 1] = *reinterpret_cast<const float2 *>(xg + b + 16);
-                    if (NORM) {
-                        nw[NORM ? p : 0][t] = *reinterpret_cast<const float2 *>(wg + b);
-                        nw[NORM ? p : 0][t + 1] = *reinterpret_cast<const float2 *>(wg + b + 16);
-                    }
-                }
+                fetch_task(xg + (idx >> 3) * 64, idx & 7, v[p]);
+                if (NORM) fetch_task(wg + (idx >> 3) * 64, idx & 7, nw[NORM ? p : 0]);
             }
         }
         float psq = 0.0f;
@@ -555,6 +545,8 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                 load_slot(q0[j], base + (size_t)row * row_bytes + (size_t)s * sizeof(q4_slot));
             }
         }
+        // nothing that waits for the activations may be scheduled ahead of the weight requests
+        __builtin_amdgcn_sched_barrier(0);
         // Where the results go, fetched now (indexed argument loads) so that nothing waits for them at the end.
         dst_bits = (uint64_t)a.dst[ii], res_bits = (uint64_t)a.residual[ii];
         asm volatile("" : "+s"(dst_bits));
@@ -569,6 +561,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             psq = wave_sum(psq);
             if (lane == 0) red[wave] = psq;
         }
+        float inv_norm = 1.0f;
         if (NORM) {
             float ss = 0.0f;
             float *stage = reinterpret_cast<float *>(lds + ns * SD);
@@ -599,15 +592,9 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             const float inv = rsqrtf(tot / (float)(ns * 64) + eps);
             if (STAGED) {
                 if ((int)threadIdx.x < ns * 8) {
-                    const int slot = threadIdx.x >> 3, g = threadIdx.x & 7;
+                    fetch_task(stage + (threadIdx.x >> 3) * 64, threadIdx.x & 7, v[0]);
 #pragma unroll
-                    for (int t = 0; t < 4; t += 2) {
-                        const int b = slot * 64 + xprep::group_x_index(g, 2 * t);
-                        const float2 lo = *reinterpret_cast<const float2 *>(stage + b);
-                        const float2 hi = *reinterpret_cast<const float2 *>(stage + b + 16);
-                        v[0][t] = make_float2(lo.x * inv, lo.y * inv);
-                        v[0][t + 1] = make_float2(hi.x * inv, hi.y * inv);
-                    }
+                    for (int t = 0; t < 4; t++) v[0][t] = make_float2(v[0][t].x * inv, v[0][t].y * inv);
                 }
             } else {
 #pragma unroll
@@ -618,6 +605,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                         v[p][t].y = (inv * v[p][t].y) * nw[NORM ? p : 0][t].y;
                     }
             }
+            inv_norm = inv;
         }
         // the corrections live behind the slots (and behind the staged activations, which other threads may still read)
         uint32_t *const corr = lds + ns * SD + (STAGED ? ns * 64 : 0);
@@ -626,9 +614,28 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             const int idx = threadIdx.x + p * THREADS;
             if (idx < ns * 8) {
                 const int slot = idx >> 3, g = idx & 7;
-                float x8[8] = {v[p][0].x, v[p][1].x, v[p][0].y, v[p][1].y,
-                               v[p][2].x, v[p][3].x, v[p][2].y, v[p][3].y};
-                prep_store<L>(x8, lds + slot * SD, corr + slot * slot_lds<L>::corr_dwords, g);
+                const float x8[8] = GH_TASK_X8(v[p]);
+                prep_store<L>(x8, lds + slot * SD, corr + slot * slot_lds<L>::corr_dwords, g, [&](float (&y8)[8]) {
+                    // the same values by the same arithmetic as above
+                    float2 w[4];
+                    if (STAGED) {
+                        fetch_task(reinterpret_cast<const float *>(lds + ns * SD) + slot * 64, g, w);
+#pragma unroll
+                        for (int t = 0; t < 4; t++) w[t] = make_float2(w[t].x * inv_norm, w[t].y * inv_norm);
+                    } else {
+                        fetch_task(xg + slot * 64, g, w);
+                        if (NORM) {
+                            float2 gw[4];
+                            fetch_task(wg + slot * 64, g, gw);
+#pragma unroll
+                            for (int t = 0; t < 4; t++)
+                                w[t] = make_float2((inv_norm * w[t].x) * gw[t].x, (inv_norm * w[t].y) * gw[t].y);
+                        }
+                    }
+                    const float t8[8] = GH_TASK_X8(w);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) y8[j] = t8[j];
+                });
             }
         }
     }

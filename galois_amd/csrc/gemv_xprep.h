@@ -10,13 +10,15 @@
 // holds exactly in integer arithmetic; the only rounding is that of x to XBITS-1 fractional
 // bits below its block's leading power of two (2^-21 relative for 6 limbs).
 //
-// What the rounding drops is not lost.  The residual r = x - X * 2^(e-XBITS+1) is exact in f32.  Activations in
-// the block's top binade (|x| >= 2^e) keep XBITS-1 bits, |r| <= 2^(1-XBITS) |x|; the others share what the common
-// scale leaves them.  A block in which the residuals of those others add up to more than 2^-15 of their sum of |x|
-// (one in which a few activations tower over the rest, so that the rest keeps few bits, or none) gets a correction
-// block: the residuals of those others in the same fixed-point form with their own scale and CORR_L limbs.  The
-// kernel adds dot(weights, correction planes) for such blocks, which takes them to 2^-13 of the largest residual
-// (at most 2^-31 of the block's largest activation); in every other block  sum_{k below the top binade} |r_k| <= 2^-15 * sum_{k below the top binade} |x_k|.
+// What the rounding drops is not lost.  The residual r = x - X * 2^(e-XBITS+1) is exact in f32 and at most half a
+// grid step, 2^(e-XBITS).  That is 2^(1-XBITS) of a block's largest activation, but it can be all of a small one:
+// a block in which one activation towers over the rest leaves the rest few bits, or none.  The decision is made on
+// the sum of |x| over the block without its largest activation: if that sum is below 31 half steps times 2^14, the
+// block gets a correction block -- the residuals of its activations below the top binade, in the same fixed-point
+// form with their own scale and CORR_L limbs -- and the kernel adds dot(weights, correction planes) for it, which
+// takes those activations to 2^-13 of their largest residual (at most 2^-31 of the block's largest activation).
+// In every other block the activations other than the largest satisfy  sum |r_k| <= 2^-14 * sum |x_k|.
+// A block too small for a grid of its own (largest activation below 2^-108) lives in its correction block alone.
 //
 // Plain C++ (no HIP builtins) so the same code is unit-tested on the CPU.
 #pragma once
@@ -95,16 +97,20 @@ GH_HD float residual(float x, float mult, float scale) {
     return __builtin_fmaf(-X, scale, x);
 }
 
-constexpr int CORR_L = 4;                              // limbs of a correction block
-constexpr float CORR_THRESHOLD = 3.0517578125e-05f;    // 2^-15
+constexpr int CORR_L = 4;                       // limbs of a correction block
+constexpr float CORR_REST_FACTOR = 253952.0f;   // 31 * 2^13: 31 half grid steps times 2^14, in grid steps
 
 // Whether |x| (as f32 bits with the sign cleared) lies below the top binade of a block whose largest |x| has the
-// bits amax_bits: only such activations count in the decision below.
+// bits amax_bits: a correction block holds the residuals of such activations only (the others keep 2^(1-XBITS)).
 GH_HD bool below_top_binade(uint32_t abs_bits, uint32_t amax_bits) { return abs_bits < (amax_bits & 0x7F800000u); }
 
-// Whether a block gets a correction block, from its sums of |r| and |x| over the activations below the top binade
-// (false for a block with a NaN in it: its scale already poisons the result).
-GH_HD bool needs_correction(float sum_abs_r, float sum_abs_x) { return sum_abs_r > CORR_THRESHOLD * sum_abs_x; }
+// Whether a block gets a correction block: sum_abs_x is the block's sum of |x|, amax_bits its largest |x| and
+// scale its grid step (block_scales).  False for a block with an inf or NaN in it: its scale already poisons the
+// result.
+GH_HD bool needs_correction(float sum_abs_x, uint32_t amax_bits, float scale) {
+    const float rest = sum_abs_x - bits_f32(amax_bits);
+    return rest < CORR_REST_FACTOR * scale || (scale == 0.0f && amax_bits != 0);
+}
 
 // 8x8 nibble transpose: in[j] nibble l  ->  out[l] nibble j.
 GH_HD void transpose_nibbles(const uint32_t in[8], uint32_t out[8]) {

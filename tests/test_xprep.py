@@ -153,12 +153,15 @@ def _emulate_gemv(shim, wq, x):
             left = xb - X[32 * blk:32 * blk + 32] * float(scales[blk]) - X2[32 * blk:32 * blk + 32] * float(scales2[blk])
             top = 2.0 ** np.floor(np.log2(np.max(np.abs(xb)))) if np.any(xb) else 0.0
             low = np.abs(xb) < top
-            assert np.all(np.abs(left[~low]) <= 2.0 ** -18 * np.abs(xb[~low]))
+            if scales[blk] != 0:
+                assert np.all(np.abs(left[~low]) <= 2.0 ** -18 * np.abs(xb[~low]))
             if scales2[blk] == 0:
-                assert np.sum(np.abs(left[low])) <= 2.0 ** -15 * np.sum(np.abs(xb[low])) * (1 + 1e-6)
+                rest = np.arange(32) != int(np.argmax(np.abs(xb)))
+                assert np.sum(np.abs(left[rest])) <= 2.0 ** -14 * np.sum(np.abs(xb[rest]))
             else:
-                assert np.all(np.abs(left[low]) <= 0.5 * float(scales2[blk]))
-                assert float(scales2[blk]) <= 2.0 ** -12 * max(np.max(np.abs(xb[low])), float(scales[blk]) / 2)
+                sel = low if scales[blk] != 0 else np.ones(32, bool)
+                assert np.all(np.abs(left[sel]) <= 0.5 * float(scales2[blk]))
+                assert float(scales2[blk]) <= 2.0 ** -12 * max(np.max(np.abs(xb[sel])), float(scales[blk]) / 2)
     return y, flagged
 
 

@@ -39,25 +39,25 @@ static void slot_full(const float *x64, uint32_t *planes, float *scales, uint32_
         }
         float mult, scale;
         xprep::block_scales<L>(amax, &mult, &scale);
-        float r[4][8], sr[4], sx[4];
+        float r[4][8], sx[4];
         uint32_t rmax = 0;
+        const bool no_grid = scale == 0.0f;
         for (int t = 0; t < 4; t++) {
-            sr[t] = sx[t] = 0.0f;
+            sx[t] = 0.0f;
             for (int j = 0; j < 8; j++) {
                 const float x = x64[xprep::group_x_index(4 * blk + t, j)];
-                const bool low = mult == 0.0f || xprep::below_top_binade(xprep::f32_bits(x) & 0x7FFFFFFFu, amax);
+                const bool low = no_grid || xprep::below_top_binade(xprep::f32_bits(x) & 0x7FFFFFFFu, amax);
                 r[t][j] = low ? xprep::residual(x, mult, scale) : 0.0f;
                 const uint32_t b = xprep::f32_bits(r[t][j]) & 0x7FFFFFFFu;
-                sr[t] += xprep::bits_f32(b);
-                sx[t] += low ? __builtin_fabsf(x) : 0.0f;
+                sx[t] += __builtin_fabsf(x);
                 rmax = b > rmax ? b : rmax;
             }
         }
-        const float sum_r = (sr[0] + sr[1]) + (sr[2] + sr[3]), sum_x = (sx[0] + sx[1]) + (sx[2] + sx[3]);
+        const float sum_x = (sx[0] + sx[1]) + (sx[2] + sx[3]);
         scales2[blk] = 0.0f;
         for (int t = 0; t < 4; t++)
             for (int l = 0; l < CL; l++) planes2[l * 8 + 4 * blk + t] = 0;
-        if (xprep::needs_correction(sum_r, sum_x)) {
+        if (xprep::needs_correction(sum_x, amax, scale)) {
             float mult2;
             xprep::block_scales<CL>(rmax, &mult2, &scales2[blk]);
             for (int t = 0; t < 4; t++) {
