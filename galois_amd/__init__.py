@@ -237,6 +237,12 @@ class Device:
                                                          _ptr(v_cache), _ptr(out), n_head, head_dim, n_past, _ptr(pos),
                                                          freq_scale, theta_scale, scale))
 
+    def attn_decode_f32_static(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale,
+                               theta_scale, scale):
+        self._check(self._lib.galois_hip_attn_decode_f32_static(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),
+                                                                _ptr(v_cache), _ptr(out), n_head, head_dim, n_past,
+                                                                _ptr(pos), freq_scale, theta_scale, scale))
+
     def attn_decode_f16kv(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
                           scale):
         self._check(self._lib.galois_hip_attn_decode_f16kv(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),

@@ -326,10 +326,20 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
 }
 
 
+// Scratch of the entry point that allocates nothing: per-head counters, then the split records.  One copy per
+// device, held from the moment the library's code is loaded there until the process ends.
+constexpr int64_t AT_STATIC_HEADS = 1024;
+constexpr int64_t AT_STATIC_FLOATS = 1 << 18;  // records: n_head * splits * (head_dim + 4) floats, 1 MB
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[AT_STATIC_HEADS * sizeof(unsigned) + AT_STATIC_FLOATS * sizeof(float)];
+namespace {
+
+// static_scratch: the partial results and counters live in the device's copy of `scratch` (ctx->attn_static)
+// instead of the blocks the context allocated.
 template <typename CT>
 int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, CT *k_cache, CT *v_cache,
                            float *out, int32_t n_head, int32_t head_dim, int32_t n_past, const int32_t *pos,
-                           float freq_scale, float theta_scale, float scale, const char *what) {
+                           float freq_scale, float theta_scale, float scale, const char *what, bool static_scratch = false) {
     GH_REQUIRE_CTX(ctx);
     GH_REQUIRE(ctx, q && k && v && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, what);
     GH_REQUIRE(ctx, n_head > 0 && n_head <= 65535 && n_past >= 0 && n_past < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
@@ -340,12 +350,24 @@ int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, 
                GALOIS_HIP_E_ALIGN, "attn_decode: 16-byte aligned vectors and caches");
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
-    GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && (int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr && ctx->attn_done != nullptr),
-               GALOIS_HIP_E_UNSUPPORTED, "attn_decode: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
-                                         "results must fit the context's 4 MB scratch block");
+    float *part;
+    unsigned *done;  // one counter per head, zero between calls
+    if (static_scratch) {
+        GH_REQUIRE(ctx, ctx->attn_static != nullptr, GALOIS_HIP_E_UNSUPPORTED, "attn_decode: the device's static scratch was not found");
+        GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && n_head <= AT_STATIC_HEADS &&
+                                   (int64_t)n_head * S * (head_dim + 4) <= AT_STATIC_FLOATS),
+                   GALOIS_HIP_E_SHAPE, "attn_decode_f32_static: at most 1024 heads and n_head * ceil((n_past + 1) / 128) * "
+                                       "(head_dim + 4) <= 262144 floats of partial results (the static 1 MB block)");
+        done = (unsigned *)ctx->attn_static;
+        part = (float *)((unsigned char *)ctx->attn_static + AT_STATIC_HEADS * sizeof(unsigned));
+    } else {
+        GH_REQUIRE(ctx, S == 1 || (S <= AT_MAX_SPLITS && (int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS && ctx->scratch != nullptr && ctx->attn_done != nullptr),
+                   GALOIS_HIP_E_UNSUPPORTED, "attn_decode: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
+                                             "results must fit the context's 4 MB scratch block");
+        part = (float *)ctx->scratch;
+        done = ctx->attn_done;
+    }
     GH_BIND(ctx);
-    float *part = (float *)ctx->scratch;
-    unsigned *done = ctx->attn_done;  // one counter per head, zero between calls
     const dim3 grid((unsigned)S, (unsigned)n_head), block(AT_THREADS);
     if (head_dim == 128)
         hipLaunchKernelGGL((attn_decode_partial<32, CT>), grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done,
@@ -357,6 +379,24 @@ int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, 
 }
 
 }  // namespace
+
+// Called by galois_hip_create with the context's device current: where this device keeps its copy of `scratch`.
+// (In host code the array's name is a handle for this lookup, not a device address.)
+int32_t gh_attn_static_init(galois_hip_ctx *ctx) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipGetSymbolAddress(attention scratch)");
+    ctx->attn_static = p;
+    return GALOIS_HIP_OK;
+}
+
+extern "C" int32_t galois_hip_attn_decode_f32_static(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
+                                                     float *k_cache, float *v_cache, float *out, int32_t n_head,
+                                                     int32_t head_dim, int32_t n_past, const int32_t *pos,
+                                                     float freq_scale, float theta_scale, float scale) {
+    return attn_decode_launch<float>(ctx, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale,
+                                     theta_scale, scale, "attn_decode_f32_static", true);
+}
 
 extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
                                               float *k_cache, float *v_cache, float *out, int32_t n_head,

@@ -15,6 +15,7 @@ struct galois_hip_ctx {
     size_t ws_bytes;
     void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul, partial results of the decode attention
     unsigned *attn_done;  // GH_ATTN_HEADS counters of the decode attention (splits finished per head), zero between calls
+    void *attn_static;    // this device's copy of the decode attention's static scratch (attn_decode.hip), found at creation
     bool capturing;   // between graph_begin_capture and graph_end_capture: nothing may allocate or block
     char last_error[256];
 };
@@ -71,5 +72,8 @@ static inline int32_t gh_hip(galois_hip_ctx *ctx, hipError_t e, const char *what
     } while (0)
 
 #define GH_LAUNCH_CHECK(ctx, what) return gh_hip((ctx), hipGetLastError(), (what))
+
+// attn_decode.hip: looks up the device's copy of the attention's static scratch (the context's device is current).
+int32_t gh_attn_static_init(galois_hip_ctx *ctx);
 
 static inline bool gh_aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }

@@ -39,6 +39,7 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     ctx->ws_bytes = 0;
     ctx->scratch = nullptr;
     ctx->attn_done = nullptr;
+    ctx->attn_static = nullptr;
     ctx->capturing = false;
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
@@ -51,6 +52,7 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     if (e == hipSuccess) e = hipMalloc((void **)&ctx->attn_done, GH_ATTN_HEADS * sizeof(unsigned));
     if (e == hipSuccess) e = hipMemsetAsync(ctx->attn_done, 0, GH_ATTN_HEADS * sizeof(unsigned), ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess && gh_attn_static_init(ctx) != GALOIS_HIP_OK) e = hipErrorNotFound;
     if (e != hipSuccess) {
         if (ctx->scratch) (void)hipFree(ctx->scratch);
         if (ctx->attn_done) (void)hipFree(ctx->attn_done);

@@ -238,6 +238,20 @@ int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const fl
                                    float *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
                                    const int32_t *pos, float freq_scale, float theta_scale, float scale);
 
+/* galois_hip_attn_decode_f32 for callers that cannot allocate device memory or have it allocated on their behalf
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and bit-identical results; the partial results and per-head counters live in a static
+ * device array of the library (1 MB + 4 KB, one copy per GPU, held until the process ends) instead of the block the
+ * context allocated at creation, and the call allocates and frees nothing.  Limits (GALOIS_HIP_E_SHAPE beyond them):
+ * n_head <= 1024 and n_head * ceil((n_past + 1) / 128) * (head_dim + 4) <= 262144, e.g. 32 heads of 128 up to
+ * 7936 cached positions.  Every context on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ * contexts, two streams) race; calls on one context are ordered by its stream.  The counters are zero when the
+ * library is loaded and every call returns them to zero. */
+int32_t galois_hip_attn_decode_f32_static(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
+                                          float *k_cache, float *v_cache, float *out, int32_t n_head, int32_t head_dim,
+                                          int32_t n_past, const int32_t *pos, float freq_scale, float theta_scale,
+                                          float scale);
+
 /* The same with f16 caches, the form the reference keeps them in on the GPU (cpy_f32_f16 into the cache,
  * src/cuda.rs:1382-1595, then gemm_ex on F16 operands, src/cuda.rs:881-992): k_cache, v_cache are
  * [n_ctx][n_head * head_dim] f16; row n_past receives rope(k) and v rounded to nearest even, and this step's scores
