@@ -197,11 +197,18 @@ def decode_step_bench(dev, reps, with_graph=True):
     tok, n_past = 1, c - 1
     res = {"config": "32 layers, d_model 4096, 32 heads, FFN 11008, vocab 32000, KV length %d, f32 cache" % c,
            "algorithmic_bytes_per_token": weight_bytes + kv_bytes, "setup_s": round(setup_s, 1)}
+    plan_logits = {}
+
+    def cross(a, b):  # max |a - b| / max |b| and relative L2 of two sets of logits
+        return {"max_rel": float(np.max(np.abs(a - b)) / np.max(np.abs(b))),
+                "l2_rel": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
+
     for name, fused in (("eager_one_kernel_per_op", 0), ("eager_fused_norm_and_silu", 1), ("eager_grouped_gemv", 2),
                         ("eager_grouped_gemv_fused_attention", 3), ("eager_split_norms", 4)):
         dec.time_steps(tok, n_past, fused, 3)
         ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
         res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
+        plan_logits[fused] = dec.logits().astype(np.float64)
     if not with_graph:
         dec.close()
         return res
@@ -214,6 +221,14 @@ def decode_step_bench(dev, reps, with_graph=True):
                               "hbm_frac": round((weight_bytes + kv_bytes) / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     logits = dec.logits()
     res["logits_finite"] = bool(np.all(np.isfinite(logits)))
+    # the 32-layer logits of the fused plans and of the graph replay against the one-kernel-per-op plan (every op its
+    # own launch, each of them parity-tested against the oracle at these shapes): the bar is the matvec's 1e-4
+    res["logits_vs_one_kernel_per_op"] = {
+        "grouped_gemv_fused_attention": cross(plan_logits[3], plan_logits[0]),
+        "split_norms": cross(plan_logits[4], plan_logits[0]),
+        "hip_graph_split_norms": cross(logits.astype(np.float64), plan_logits[0])}
+    res["logits_within_1e-4"] = bool(all(v["max_rel"] < 1e-4 and v["l2_rel"] < 1e-4
+                                         for v in res["logits_vs_one_kernel_per_op"].values()))
     dec.close()
     # the same step with the KV cache in f16 (the form the reference keeps it in on the GPU): half the cache bytes
     dec, _ = make_decoder(True)

@@ -228,8 +228,9 @@ class Device:
         self._check(self._lib.galois_hip_cpy_f32(self._ctx, _ptr(x), _ptr(dst), int(dst_is_f16), ne, ne00, ne01, nb00,
                                                  nb01, nb02, ne10, ne11, nb10, nb11, nb12))
 
-    def get_rows_q4_0(self, table, ids, dst, ncols, nr):
-        self._check(self._lib.galois_hip_get_rows_q4_0(self._ctx, _ptr(table), _ptr(ids), _ptr(dst), ncols, nr))
+    def get_rows_q4_0(self, table, ids, dst, ncols, nr, n_table_rows):
+        self._check(self._lib.galois_hip_get_rows_q4_0(self._ctx, _ptr(table), _ptr(ids), _ptr(dst), ncols, nr,
+                                                       n_table_rows))
 
     def attn_decode_f32(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
                         scale):

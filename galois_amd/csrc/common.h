@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <vector>
+
 #include "../../include/galois_hip.h"
 
 struct galois_hip_ctx {
@@ -13,6 +15,7 @@ struct galois_hip_ctx {
     int32_t n_cu;
     void *ws;         // workspace owned by the context (fp16 activations of the prefill matmul)
     size_t ws_bytes;
+    std::vector<void *> ws_retired;  // outgrown workspaces: a graph captured earlier may still point into them
     void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul, partial results of the decode attention
     unsigned *attn_done;  // GH_ATTN_HEADS counters of the decode attention (splits finished per head), zero between calls
     void *attn_static;    // this device's copy of the decode attention's static scratch (attn_decode.hip), found at creation

@@ -69,6 +69,7 @@ int32_t galois_hip_destroy(galois_hip_ctx *ctx) {
     (void)hipSetDevice(ctx->ordinal);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    for (void *p : ctx->ws_retired) (void)hipFree(p);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->attn_done) (void)hipFree(ctx->attn_done);
     hipError_t e = hipStreamDestroy(ctx->stream);

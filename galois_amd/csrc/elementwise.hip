@@ -88,15 +88,22 @@ __global__ __launch_bounds__(kEwThreads) void cpy_strided(const char *__restrict
 }
 
 // get_rows for a Q4_0 table (GetRows::f_q_x_f32, src/op.rs:2546-2571; CPU-only in the reference):
-// dst row i = to_f32(table row ids[i]).  One wave per row, one block per lane per step.
+// dst row i = to_f32(table row ids[i]).  One wave per row, one block per lane per step.  The ids come from device
+// memory, so they are checked here: a row whose id is outside the table is filled with NaN and no table byte is
+// read for it (the reference indexes bounded slices and would panic).
 __global__ __launch_bounds__(kEwThreads) void get_rows_q4_0(const uint16_t *__restrict__ table,
                                                             const int32_t *__restrict__ ids, float *__restrict__ dst,
-                                                            int nblocks, int nr) {
+                                                            int nblocks, int nr, int n_table_rows) {
     const int lane = threadIdx.x & 63;
     const int r = blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
     if (r >= nr) return;
-    const uint16_t *row = table + (size_t)ids[r] * nblocks * 9;
+    const int id = ids[r];
     float *out = dst + (size_t)r * nblocks * 32;
+    if (id < 0 || id >= n_table_rows) {  // wave-uniform
+        for (int i = lane; i < nblocks * 32; i += 64) out[i] = __builtin_nanf("");
+        return;
+    }
+    const uint16_t *row = table + (size_t)id * nblocks * 9;
     for (int b = lane; b < nblocks; b += 64) {
         const uint16_t *p = row + (size_t)b * 9;
         const float d = (float)__builtin_bit_cast(_Float16, p[0]);
@@ -211,14 +218,14 @@ int32_t galois_hip_cpy_f32(galois_hip_ctx *ctx, const void *x, void *dst, int32_
 }
 
 int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const int32_t *ids, float *dst, int32_t ncols,
-                                 int32_t nr) {
+                                 int32_t nr, int32_t n_table_rows) {
     GH_REQUIRE_CTX(ctx);
     GH_REQUIRE(ctx, table && ids && dst, GALOIS_HIP_E_NULL, "get_rows_q4_0");
-    GH_REQUIRE(ctx, ncols > 0 && ncols % 32 == 0 && nr > 0, GALOIS_HIP_E_SHAPE, "get_rows_q4_0");
+    GH_REQUIRE(ctx, ncols > 0 && ncols % 32 == 0 && nr > 0 && n_table_rows > 0, GALOIS_HIP_E_SHAPE, "get_rows_q4_0");
     GH_REQUIRE(ctx, gh_aligned(table, 2) && gh_aligned(ids, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "get_rows_q4_0");
     GH_BIND(ctx);
     hipLaunchKernelGGL(get_rows_q4_0, dim3((nr + 3) / 4), dim3(kEwThreads), 0, ctx->stream, (const uint16_t *)table,
-                       ids, dst, ncols / 32, nr);
+                       ids, dst, ncols / 32, nr, n_table_rows);
     GH_LAUNCH_CHECK(ctx, "get_rows_q4_0 launch");
 }
 

@@ -304,11 +304,6 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
     uint8_t *raw0 = reinterpret_cast<uint8_t *>(smem + GNBUF * GB_HALFS);
     uint8_t *raw1 = raw0 + GRAW_BYTES;
 
-#ifdef GEMM_X_NO_PROD
-    __syncthreads();
-    for (int t = 0; t < nslots; t++) __syncthreads();
-    return;
-#endif
     gemm_raw_regs<GN> rr;
     gemm_load_raw(W, wrow_bytes, N, n0, p, 0, rr);
     GEMM_VMWAIT(0);
@@ -372,29 +367,8 @@ __device__ __forceinline__ void gemm_load_a1(u32x4_t &dst, const _Float16 *xs, u
                  : "+v"((r).c[0]), "+v"((r).c[1]), "+v"((r).c[2]), "+v"((r).c[3]), "+v"((r).c[4]), "+v"((r).c[5]), \
                    "+v"((r).c[6]), "+v"((r).c[7])::"memory")
 
-// Tuning builds: -DGEMM_X_NO_A / _NO_B / _NO_MFMA / _NO_PROD / _NO_STORE compile the kernel without its A
-// requests, B fragment reads, matrix instructions, producer work or result store (results are then
-// meaningless) to time what each part costs.
-#ifdef GEMM_X_NO_A
-#define GEMM_XA(...)
-#else
-#define GEMM_XA(...) __VA_ARGS__
-#endif
-#ifdef GEMM_X_NO_B
-#define GEMM_LDB(dst, ptr) asm volatile("" : "+v"(dst))
-#else
 #define GEMM_LDB(dst, ptr) dst = *reinterpret_cast<const half8_t *>(ptr)
-#endif
-#ifdef GEMM_X_NO_MFMA
-#define GEMM_MFMA(a, b, c) (c)
-#else
 #define GEMM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
-#endif
-#ifdef GEMM_X_NO_MFMA
-#define GEMM_XKEEP _Pragma("unroll") for (int j = 0; j < NF; j++) { asm volatile("" ::"v"(b0[j]), "v"(b1[j])); }
-#else
-#define GEMM_XKEEP
-#endif
 template <int NF, int GN>
 __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float16 *__restrict__ Xh,
                                               float *__restrict__ Y, int K, int N, int M, int m0, int n0, int wm,
@@ -416,13 +390,11 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
 
     gemm_a_regs a0, a1;
     // requested in the order they are used: the waits below count younger requests
-    GEMM_XA(_Pragma("unroll") for (int g = 0; g < 8; g++) gemm_load_a1(a0.c[g], Xh, ro[g & 3], g >> 2);)
-    GEMM_XA(_Pragma("unroll") for (int g = 0; g < 8; g++) gemm_load_a1(a1.c[g], Xh + 1024, ro[g & 3], g >> 2);)
-    half8_t b0[NF], b1[NF];
-#ifdef GEMM_X_NO_B
 #pragma unroll
-    for (int j = 0; j < NF; j++) b1[j] = half8_t{1, 1, 1, 1, 1, 1, 1, 1};
-#endif
+    for (int g = 0; g < 8; g++) gemm_load_a1(a0.c[g], Xh, ro[g & 3], g >> 2);
+#pragma unroll
+    for (int g = 0; g < 8; g++) gemm_load_a1(a1.c[g], Xh + 1024, ro[g & 3], g >> 2);
+    half8_t b0[NF], b1[NF];
     __syncthreads();  // R
     __syncthreads();  // stage 0 written
 #pragma unroll
@@ -441,12 +413,12 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
     constexpr int BPG = (NF + 2) / 3;  // B fragment reads per group
 #define GEMM_GROUP(G, AC, BV)                                                                              \
     {                                                                                                      \
-        GEMM_XA(asm volatile("s_waitcnt vmcnt(15)" : "+v"((AC).c[G])::"memory");)                          \
+        asm volatile("s_waitcnt vmcnt(15)" : "+v"((AC).c[G])::"memory");                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                 \
         _Pragma("unroll") for (int j = 0; j < NF; j++) acc[(G) & 3][j] =                                   \
             GEMM_MFMA(__builtin_bit_cast(half8_t, (AC).c[G]), BV[j], acc[(G) & 3][j]);                     \
         __builtin_amdgcn_sched_barrier(0);                                                                 \
-        GEMM_XA(gemm_load_a1((AC).c[G], xs_next, ro[(G) & 3], (G) >> 2);)                                  \
+        gemm_load_a1((AC).c[G], xs_next, ro[(G) & 3], (G) >> 2);                                           \
     }
 #define GEMM_BREADS(G3, DST, OFF)                                                                          \
     _Pragma("unroll") for (int j = (G3) * BPG; j < NF && j < ((G3) + 1) * BPG; j++)                        \
@@ -468,7 +440,6 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
         if (!(LAST)) { GEMM_BREADS(2, b0, nxt) }                                                           \
         GEMM_GROUP(6, AC, b1)                                                                              \
         GEMM_GROUP(7, AC, b1)                                                                              \
-        GEMM_XKEEP                                                                                         \
         cur = nxt;                                                                                         \
         nxt = (nxt == b_off + (GNBUF - 1) * GB_HALFS) ? b_off : nxt + GB_HALFS;                            \
     }
@@ -483,7 +454,8 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
 #undef GEMM_GROUP
 #undef GEMM_BREADS
     // the last two stages requested the last stage's fragments again (never used): drain before the registers die
-    GEMM_XA(GEMM_DRAIN_A(a0); GEMM_DRAIN_A(a1);)
+    GEMM_DRAIN_A(a0);
+    GEMM_DRAIN_A(a1);
 
     // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e
 #pragma unroll
@@ -494,11 +466,7 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + e;
-#ifdef GEMM_X_NO_STORE
-                if (m < M && n < N && acc[i][j][e] == 1234.5f) Y[(size_t)m * N + n] = acc[i][j][e];
-#else
                 if (m < M && n < N) Y[(size_t)m * N + n] = acc[i][j][e];
-#endif
             }
         }
 }
@@ -522,19 +490,17 @@ __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict_
         gemm_consumer<GN / 16, GN>(smem, Xh, Y, K, N, M, m0, n0, wave, 0);
 }
 
-// Launch of one tile width; the attribute that lifts the dynamic LDS limit is set once per instantiation.
+// Launch of one tile width.
 template <int GN>
 int32_t gemm_launch(galois_hip_ctx *ctx, const uint8_t *W, const _Float16 *Xh, float *Y, int K, int N, int M) {
     const int n_tiles = (N + GN - 1) / GN, m_tiles = (M + GM - 1) / GM;
     const int total = n_tiles * m_tiles;
     const int grid = ((total + 7) / 8) * 8;
     const size_t lds = gemm_cfg<GN>::LDS_BYTES;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_q4_0_mfma<GN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
-        attr_set = true;
-    }
+    // the attribute lives with the function on the current device: set per launch (a table lookup), which is right
+    // for every device and every thread without any flag of our own
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_q4_0_mfma<GN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
     hipLaunchKernelGGL(gemm_q4_0_mfma<GN>, dim3(grid), dim3(512), lds, ctx->stream, W, Xh, Y, K, N, M, n_tiles, m_tiles);
     return GALOIS_HIP_OK;
 }
@@ -551,20 +517,20 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
                "mul_mat_q4_0_f32: W 2-byte, X 16-byte, Y 4-byte aligned");
     GH_BIND(ctx);
     if (K % 256 == 0 && gh_aligned(W, 16) && ((int64_t)M + 16) * K * 2 < ((int64_t)1 << 32)) {
-        // fp16 copy of X, tiled for the A fragments, in the context's workspace (grown on demand, kept
-        // until the context dies)
+        // fp16 copy of X, tiled for the A fragments, in the context's workspace (grown on demand)
         const int64_t m_pad = ((int64_t)M + 15) / 16 * 16;
         const size_t need = (size_t)m_pad * K * sizeof(_Float16);
         if (ctx->ws_bytes < need) {
             GH_NOT_CAPTURING(ctx, "mul_mat_q4_0_f32: growing the fp16 workspace");
-            hipError_t e = hipStreamSynchronize(ctx->stream);
-            if (e != hipSuccess) return gh_hip(ctx, e, "hipStreamSynchronize");
-            if (ctx->ws) (void)hipFree(ctx->ws);
-            ctx->ws = nullptr;
-            ctx->ws_bytes = 0;
-            e = hipMalloc(&ctx->ws, need);
+            // The outgrown block is kept until the context dies: work already queued, or a graph captured earlier,
+            // has its address baked in.  Growing by at least half bounds what the retired blocks add up to.
+            const size_t bytes = need > ctx->ws_bytes + ctx->ws_bytes / 2 ? need : ctx->ws_bytes + ctx->ws_bytes / 2;
+            void *grown = nullptr;
+            const hipError_t e = hipMalloc(&grown, bytes);
             if (e != hipSuccess) return gh_hip(ctx, e, "hipMalloc(workspace)");
-            ctx->ws_bytes = need;
+            if (ctx->ws) ctx->ws_retired.push_back(ctx->ws);
+            ctx->ws = grown;
+            ctx->ws_bytes = bytes;
         }
         _Float16 *Xh = (_Float16 *)ctx->ws;
         const int64_t nchunks = m_pad * K / 8;

@@ -241,6 +241,8 @@ GResult galois_rms_norm(const Tensor &src, Tensor &dst, float eps) {
     if (src.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32) return err(GError::Unimplemented, "galois_rms_norm: F32 only");
     if (src.dim().elem_count() != dst.dim().elem_count() || src.dim().shape[0] != dst.dim().shape[0])
         return err(GError::ShapeError, "rms_norm: src and dst shapes differ");
+    if (!src.dim().ggml_is_contiguous(src.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_rms_norm: contiguous operands only (the kernel walks whole rows)");
     return dev->check(galois_hip_rms_norm_f32(dev->ctx(), (const float *)src.data(), (float *)dst.data(),
                                               (int32_t)src.dim().shape[0], (int32_t)src.dim().nrows(), eps));
 }
@@ -258,6 +260,8 @@ GResult galois_rope_custom(const RopeCustomOption &op, const Tensor &src0, const
     if (op.n_dims == 0 || op.n_dims % 2 != 0 || src0.dim().shape[0] % 2 != 0)
         return err(GError::ShapeError, "rope: n_dims and ne00 must be even");
     if (src0.dim().elem_count() != dst.dim().elem_count()) return err(GError::ShapeError, "rope: src and dst shapes differ");
+    if (!src0.dim().ggml_is_contiguous(src0.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_rope_custom: contiguous operands only (the kernel walks whole rows)");
     const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);  // src/cuda.rs:1327
     return dev->check(galois_hip_rope_f32(dev->ctx(), (const float *)src0.data(), (float *)dst.data(),
                                           (int32_t)src0.dim().shape[0], (int32_t)src0.dim().nrows(),
@@ -272,6 +276,8 @@ GResult galois_soft_max(const Tensor &src, Tensor &dst) {
     if (src.dtype() != GGmlType::F32 || dst.dtype() != GGmlType::F32) return err(GError::Unimplemented, "soft_max: F32 only");
     if (src.dim().elem_count() != dst.dim().elem_count() || src.dim().shape[0] != dst.dim().shape[0])
         return err(GError::ShapeError, "soft_max: src and dst shapes differ");
+    if (!src.dim().ggml_is_contiguous(src.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_soft_max: contiguous operands only (the kernel walks whole rows)");
     return dev->check(galois_hip_soft_max_f32(dev->ctx(), (const float *)src.data(), (float *)dst.data(),
                                               (int32_t)src.dim().shape[0], (int32_t)src.dim().nrows()));
 }
@@ -357,7 +363,7 @@ GResult galois_get_rows(const Tensor &src0, const Tensor &src1, Tensor &dst) {
     if (!src0.dim().ggml_is_contiguous(src0.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()))
         return err(GError::Unimplemented, "galois_get_rows: contiguous operands only");
     return dev->check(galois_hip_get_rows_q4_0(dev->ctx(), src0.data(), (const int32_t *)src1.data(), (float *)dst.data(),
-                                               (int32_t)nc, (int32_t)nr));
+                                               (int32_t)nc, (int32_t)nr, (int32_t)src0.dim().shape[1]));
 }
 
 }  // namespace galois

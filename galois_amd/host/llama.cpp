@@ -22,6 +22,9 @@ GResult galois_rms_norm_mul(const Tensor &src, const Tensor &weight, Tensor &dst
         return err(GError::Unimplemented, "galois_rms_norm_mul: F32 only");
     if (weight.dim().elem_count() != src.dim().shape[0] || src.dim().elem_count() != dst.dim().elem_count())
         return err(GError::ShapeError, "rms_norm_mul: weight must have ne00 elements, dst the shape of src");
+    if (!src.dim().ggml_is_contiguous(src.dtype()) || !dst.dim().ggml_is_contiguous(dst.dtype()) ||
+        !weight.dim().ggml_is_contiguous(weight.dtype()))
+        return err(GError::Unimplemented, "galois_rms_norm_mul: contiguous operands only (the kernel walks whole rows)");
     const auto &dev = src.device().gpu;
     return dev->check(galois_hip_rms_norm_mul_f32(dev->ctx(), (const float *)src.data(), (const float *)weight.data(),
                                                   (float *)dst.data(), (int32_t)src.dim().shape[0],
@@ -196,6 +199,10 @@ GResult LlamaDecoder::set_inputs(int32_t token, int32_t n_past) {
 GResult LlamaDecoder::step(int32_t n_past, int fused) {
     if (hp_.kv_f16 && fused < 3)
         return err(GError::Unimplemented, "LlamaDecoder: an f16 KV cache runs with the fused attention only (fused = 3)");
+    // the grouped launches take vectors of a multiple of 64 up to 12288 elements (one pass through LDS)
+    if (fused >= 2 && (hp_.n_embd % 64 != 0 || hp_.n_ff % 64 != 0 || hp_.n_embd > 12288 || hp_.n_ff > 12288))
+        return err(GError::Unimplemented, "LlamaDecoder: the grouped launch plans (fused >= 2) need n_embd and n_ff to be "
+                                          "multiples of 64 no larger than 12288; use fused = 0 or 1");
     const size_t E = hp_.n_embd, H = hp_.n_head, D = E / H, L = (size_t)n_past + 1, C = hp_.n_ctx;
     RopeCustomOption rope;
     rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;

@@ -215,9 +215,11 @@ int32_t galois_hip_cpy_f32(galois_hip_ctx *ctx, const void *x, void *dst, int32_
                            int64_t ne01, int64_t nb00, int64_t nb01, int64_t nb02, int64_t ne10, int64_t ne11,
                            int64_t nb10, int64_t nb11, int64_t nb12);
 /* get_rows for a Q4_0 table: GetRows::f_q_x_f32, src/op.rs:2546-2571 (CPU-only in the reference; its GPU
- * arm is todo!(), src/op.rs:3281-3292): dst row i = to_f32(table row ids[i]), ncols % 32 == 0. */
+ * arm is todo!(), src/op.rs:3281-3292): dst row i = to_f32(table row ids[i]), ncols % 32 == 0.  The table has
+ * n_table_rows rows; the ids are read on the device, so an id outside 0 .. n_table_rows - 1 cannot be refused
+ * here: its dst row is filled with NaN and nothing is read for it (the reference's slice index would panic). */
 int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const int32_t *ids, float *dst,
-                                 int32_t ncols, int32_t nr);
+                                 int32_t ncols, int32_t nr, int32_t n_table_rows);
 /* f32 x f32 batched matmul with galois's shape conventions; todo!() in the reference (src/cuda.rs:867-879,
  * src/op.rs:1624-1662).  a = [K, N, ne02] with element strides a_s0, a_s1, a_s2 (one of a_s0, a_s1 must
  * be 1, so permuted K/V-cache views work), b = [K, M, ne12] contiguous, dst = [N, M, ne12];

@@ -77,6 +77,22 @@ q["f16_scale_rounding"] = {
     "x": [f32(v) for v in x],
     "block": block(d32, [0 if j == 17 else 8 for j in range(32)]),
 }
+# which d the reciprocal is taken of: max = -1.0003f gives d = 0.12503..., which is stored as f16 0.125; the rule takes
+# id = 1 / d from the f32 d (7.9976...), so 0.4375 -> trunc(0.4375 * id + 8.5) = trunc(11.998..) = 11, whereas a
+# reciprocal of the stored f16 d (exactly 8) would give trunc(12.0) = 12
+x = [0.0] * 32
+x[0], x[1] = f32(-1.0003), 0.4375
+d32 = f32(x[0] / -8.0)
+id32 = f32(1.0 / d32)
+q1 = int(f32(f32(x[1] * id32) + 8.5))
+q0 = int(f32(f32(x[0] * id32) + 8.5))
+d16 = struct.unpack("<e", struct.pack("<e", d32))[0]
+assert d16 == 0.125 and (q0, q1) == (0, 11) and int(f32(f32(x[1] * f32(1.0 / d16)) + 8.5)) == 12
+q["reciprocal_of_the_f32_scale"] = {
+    "why": "id = 1/d uses the unrounded f32 d: 0.4375 lands on nibble 11; 1/f16(d) = 8 would give 12",
+    "x": x,
+    "block": block(d32, [q0, q1] + [8] * 30),
+}
 cases["quantize_q4_0"] = q
 
 # --- Q8_0 KATs (BlockQ8_0::from_f32): amax=127 -> d=1, id=1, q = round-half-away(x)

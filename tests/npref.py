@@ -97,3 +97,19 @@ def rel_err(got, ref):
     den_max = max(np.max(np.abs(ref)), 1e-300)
     den_l2 = max(np.linalg.norm(ref.ravel()), 1e-300)
     return float(np.max(np.abs(d)) / den_max), float(np.linalg.norm(d.ravel()) / den_l2)
+
+
+def rope_f32_angles(x, pos, freq_scale, p_delta_rows, theta_scale):
+    """rope_f32 with the reference kernel's f32 angle (galois-kernels/src/rope.cu:16-20):
+    theta = f32(f32(pos * freq_scale) * powf(theta_scale, col / 2)), then the rotation in f64.  What is left between
+    this and an f32 kernel is the last bit of powf and of sin / cos, not the rounding of the angle itself."""
+    x = np.asarray(x, np.float32)
+    nrows, ncols = x.shape
+    p0 = (np.asarray(pos, np.int64)[np.arange(nrows) // p_delta_rows].astype(np.float32) * np.float32(freq_scale))
+    pw = np.power(np.float32(theta_scale), np.arange(ncols // 2, dtype=np.float32)).astype(np.float32)
+    theta = (p0[:, None] * pw[None, :]).astype(np.float32).astype(np.float64)
+    x0, x1 = x[:, 0::2].astype(np.float64), x[:, 1::2].astype(np.float64)
+    out = np.empty(x.shape, np.float64)
+    out[:, 0::2] = x0 * np.cos(theta) - x1 * np.sin(theta)
+    out[:, 1::2] = x0 * np.sin(theta) + x1 * np.cos(theta)
+    return out

@@ -37,6 +37,84 @@ def test_ctypes_prototypes_cover_header_exactly():
     assert sorted(_abi.PROTOTYPES) == _declared()
 
 
+def _c_prototypes():
+    """name -> (return class, [argument class, ...]) from the header text.  Classes: i32, i64, f32, size, ptr."""
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+
+    def cls(t):
+        t = t.strip()
+        if "*" in t:
+            return "ptr"
+        t = re.sub(r"\bconst\b", "", t).split()
+        base = t[0] if t[0] in ("int32_t", "int64_t", "float", "size_t") else None
+        assert base, t
+        return {"int32_t": "i32", "int64_t": "i64", "float": "f32", "size_t": "size"}[base]
+
+    out = {}
+    for ret, name, args in re.findall(r"\n((?:const\s+)?[a-z0-9_]+\s*\*?)\s*(galois_hip_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", src):
+        argl = [] if args.strip() in ("", "void") else [cls(a) for a in args.split(",")]
+        out[name] = (cls(ret), argl)
+    return out
+
+
+def _ctypes_class(t):
+    if t in (C.c_int32,):
+        return "i32"
+    if t in (C.c_int64,):
+        return "i64"
+    if t is C.c_float:
+        return "f32"
+    if t is C.c_size_t:
+        return "size"
+    return "ptr"  # c_void_p, c_char_p, POINTER(...)
+
+
+def test_ctypes_argument_lists_match_the_header():
+    cproto = _c_prototypes()
+    assert sorted(cproto) == _declared()
+    for name, (res, args) in _abi.PROTOTYPES.items():
+        cres, cargs = cproto[name]
+        assert [_ctypes_class(a) for a in args] == cargs, name
+        assert _ctypes_class(res) == cres, name
+
+
+def _rust_prototypes():
+    """The extern block of INTEGRATION.md, the binding a maintainer would paste into src/hip.rs."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    out = {}
+    for name, args, ret in re.findall(r"pub fn (galois_hip_[a-z0-9_]+)\(([^)]*)\)\s*->\s*([^;]+);", text):
+        def cls(t):
+            t = t.split(":", 1)[1].strip()
+            if t.startswith("*"):
+                return "ptr"
+            return {"i32": "i32", "i64": "i64", "f32": "f32", "usize": "size"}[t]
+        argl = [cls(a) for a in args.split(",") if a.strip()]
+        out[name] = ("ptr" if ret.strip().startswith("*") else {"i32": "i32"}[ret.strip()], argl)
+    return out
+
+
+def test_rust_binding_block_matches_the_header():
+    rust, cproto = _rust_prototypes(), _c_prototypes()
+    assert sorted(rust) == sorted(cproto), sorted(set(cproto) ^ set(rust))
+    for name, sig in rust.items():
+        assert sig == cproto[name], name
+    # the struct of the grouped launch, field for field
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    body = re.search(r"pub struct GaloisHipGemvItem \{(.*?)\}", text, flags=re.S).group(1)
+    body = re.sub(r"//[^\n]*", "", body)
+    rust_fields = [f.strip().split(":")[0].replace("pub ", "").strip() for f in body.replace("\n", " ").split(",") if ":" in f]
+    assert rust_fields == [f[0] for f in _abi.GemvItem._fields_]
+    hsrc = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    cbody = re.search(r"typedef struct galois_hip_gemv_item \{(.*?)\}", hsrc, flags=re.S).group(1)
+    c_fields = []
+    for decl in cbody.split(";"):
+        decl = decl.strip()
+        if decl:
+            c_fields += [re.sub(r"[*\s]", "", n.split()[-1]) for n in decl.split(",")]
+    assert c_fields == rust_fields
+
+
 def test_status_strings_without_device():
     lib = _abi.load()
     assert lib.galois_hip_status_string(0) == b"ok"

@@ -62,7 +62,10 @@ def _run(dev, q, k, v, kc, vc, H, D, n_past, fs, ts, scale):
 
 @pytest.mark.parametrize("H,D,n_ctx,n_past", [(32, 128, 2048, 2047), (32, 128, 2048, 0), (32, 128, 300, 127),
                                               (32, 128, 300, 128), (32, 128, 300, 129), (3, 128, 700, 511),
-                                              (2, 64, 64, 37), (5, 64, 1000, 999), (1, 64, 130, 1)])
+                                              (2, 64, 64, 37), (5, 64, 1000, 999), (1, 64, 130, 1),
+                                              # more than 16 splits: the merge that keeps its weights in LDS
+                                              # (17, 40 and 313 splits; past 256 its loops go round twice)
+                                              (32, 128, 2049, 2048), (8, 128, 5001, 5000), (2, 64, 40001, 40000)])
 def test_attn_decode_matches_the_op_sequence(dev, H, D, n_ctx, n_past):
     rng = np.random.default_rng(H * 1000 + D + n_past)
     E = H * D
@@ -85,10 +88,11 @@ def test_attn_decode_matches_the_op_sequence(dev, H, D, n_ctx, n_past):
     assert np.array_equal(vc_g[n_past], v)
     assert np.array_equal(kc_g[n_past], kr)
     emax, _ = npref.rel_err(kc_g[n_past], kc_ref[n_past])
-    assert emax < TOL_ROPE
+    assert emax < TOL_ROPE * max(1.0, n_past / 2048.0)   # the f32 angle's rounding grows with the position
 
 
-@pytest.mark.parametrize("H,D,n_ctx,n_past", [(32, 128, 2048, 2047), (32, 128, 300, 128), (2, 64, 64, 37), (5, 64, 1000, 0)])
+@pytest.mark.parametrize("H,D,n_ctx,n_past", [(32, 128, 2048, 2047), (32, 128, 300, 128), (2, 64, 64, 37), (5, 64, 1000, 0),
+                                              (4, 128, 2200, 2100), (2, 64, 34000, 33500)])
 def test_attn_decode_with_f16_caches(dev, H, D, n_ctx, n_past):
     """f16 caches: the appended rows are rope(k) and v rounded to nearest even, and the step computes with the
     rounded rows, like cpy_f32_f16 into the cache followed by the matmuls on its f16 contents."""
@@ -134,10 +138,11 @@ def test_attn_decode_invariants(dev):
     assert emax < TOL and el2 < TOL
 
 
-def test_attn_decode_repeated_calls_merge_fresh_partials(dev):
+@pytest.mark.parametrize("L", [1500, 2700])   # 12 splits per head (merge in registers) and 22 (weights in LDS)
+def test_attn_decode_repeated_calls_merge_fresh_partials(dev, L):
     """The splits of a head are merged by whichever workgroup finishes last, reading the other workgroups' records
     from a block that every call reuses: back-to-back calls with different values must each merge their own."""
-    H, D, L = 32, 128, 1500          # 12 splits per head
+    H, D = 32, 128
     rng = np.random.default_rng(21)
     fs, ts, scale = 1.0, float(np.float32(10000.0) ** np.float32(-2.0 / D)), float(1.0 / np.sqrt(D))
     kc = rng.standard_normal((L, H * D)).astype(np.float32)

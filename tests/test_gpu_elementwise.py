@@ -70,8 +70,14 @@ def test_get_rows_q4_0(dev):
     w = oracle.quantize_q4_0((rng.standard_normal((100, 4096)) * 0.02).astype(np.float32))
     ids = np.array([99, 0, 5, 5, 42], np.int32)
     wb, ib, ob = dev.upload(w), dev.upload(ids), _out(dev, 5 * 4096)
-    dev.get_rows_q4_0(wb, ib, ob, 4096, 5)
+    dev.get_rows_q4_0(wb, ib, ob, 4096, 5, 100)
     assert np.array_equal(dev.download(ob, np.float32, (5, 4096)), oracle.get_rows_q4_0(w, ids))
+    # ids outside the table: nothing is read for them, their rows come back as NaN, the others as before
+    bad = np.array([3, 100, -1, 2 ** 31 - 1, 7], np.int32)
+    dev.upload(bad, ib)
+    dev.get_rows_q4_0(wb, ib, ob, 4096, 5, 100)
+    got = dev.download(ob, np.float32, (5, 4096))
+    assert np.array_equal(got[[0, 4]], oracle.get_rows_q4_0(w, bad[[0, 4]])) and np.all(np.isnan(got[1:4]))
 
 
 def test_attention_matmuls_over_a_kv_cache(dev):
@@ -111,7 +117,8 @@ def test_elementwise_argument_errors(dev):
     from galois_amd import GaloisHipError
     buf = dev.alloc(4096)
     for call, code in ((lambda: dev.add_f32(buf, buf, buf, 0, 1), -2), (lambda: dev.mul_f32(buf, None, buf, 4, 4), -1),
-                       (lambda: dev.get_rows_q4_0(buf, buf, buf, 48, 1), -2),
+                       (lambda: dev.get_rows_q4_0(buf, buf, buf, 48, 1, 10), -2),
+                       (lambda: dev.get_rows_q4_0(buf, buf, buf, 32, 1, 0), -2),
                        (lambda: dev.mul_mat_f32(buf, buf, buf, 4, 4, 1, 1, 1, 2, 2, 16), -5),
                        (lambda: dev.cpy_f32(buf, buf, False, 4, 2, 2, 3, 8, 16, 2, 2, 4, 8, 16), -3)):
         with pytest.raises(GaloisHipError) as ei:

@@ -107,6 +107,17 @@ def test_errors_instead_of_panics(gpu):
     assert e.value.kind == "Unimplemented"
     with pytest.raises(g.GError):        # ne0 not a multiple of the block size
         g.Tensor.zeros([48, 1], g.Q4_0, gpu)
+    # the row kernels walk contiguous rows: a permuted view is refused, not read as if it were contiguous
+    m = g.Tensor.zeros([64, 8], g.F32, gpu)
+    mt = m.view_strided(0, [8, 64], [64, 1])     # the transpose
+    out = g.Tensor.zeros([8, 64], g.F32, gpu)
+    for call in (lambda: g.galois_rms_norm(mt, out, 1e-6), lambda: g.galois_soft_max(mt, out),
+                 lambda: g.galois_soft_max(out, mt),
+                 lambda: g.galois_rope_custom({"n_dims": 8, "mode": 0}, mt.view_strided(0, [8, 64, 1], [64, 1, 512]),
+                                              g.Tensor.zeros([1], g.I32, gpu), out.view(0, [8, 64, 1]))):
+        with pytest.raises(g.GError) as e:
+            call()
+        assert e.value.kind == "Unimplemented"
     with pytest.raises(g.GError) as e:
         g.Device.gpu(999)
     assert e.value.kind == "DeviceError"

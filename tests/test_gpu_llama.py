@@ -190,20 +190,35 @@ def test_capture_refuses_calls_that_allocate_or_block(dev):
     dev.graph_destroy(graph)
 
 
-def test_full_width_layer_at_kv_length_2048(gdev):
-    """One layer at LLaMA-7B width (4096 / 32 heads / 11008 / vocab 32000) attending over 2048 cached positions."""
+def test_full_width_layers_at_kv_length_2048(gdev):
+    """Two layers at LLaMA-7B width (4096 / 32 heads / 11008 / vocab 32000) attending over 2048 cached positions,
+    through every launch plan the benchmark reports (the second layer takes the first one's residual stream and, in
+    the split-norm plan, its pre-weighted copy and partial sums of squares), a graph replay of the last plan, and the
+    f16 KV cache."""
     rng = np.random.default_rng(53)
-    hp = dict(n_vocab=32000, n_embd=4096, n_head=32, n_layer=1, n_ff=11008, n_ctx=2048, rms_eps=1e-6,
+    hp = dict(n_vocab=32000, n_embd=4096, n_head=32, n_layer=2, n_ff=11008, n_ctx=2048, rms_eps=1e-6,
               freq_base=10000.0)
     w = _make_weights(rng, hp)
-    kc = rng.standard_normal((1, 2048, 4096)).astype(np.float32)
-    vc = rng.standard_normal((1, 2048, 4096)).astype(np.float32)
+    kc = rng.standard_normal((2, 2048, 4096)).astype(np.float32)
+    vc = rng.standard_normal((2, 2048, 4096)).astype(np.float32)
     dec = g.LlamaDecoder(gdev, **hp)
+    ref = _ref_step(w, hp, kc.copy(), vc.copy(), 31999, 2047)
+    for fused in (0, 1, 2, 3, 4):
+        _load(dec, w, kc, vc)
+        dec.decode(31999, 2047, fused)
+        _check(dec.logits(), ref, 1e-4)
     _load(dec, w, kc, vc)
-    ref = _ref_step(w, hp, kc, vc, 31999, 2047)
-    dec.decode(31999, 2047, False)
-    _check(dec.logits(), ref, 1e-4)
-    dec.capture(31999, 2047, True)
-    dec.replay()
-    _check(dec.logits(), ref, 1e-4)
+    dec.capture(31999, 2047, 4)
+    for _ in range(2):
+        dec.replay()
+        _check(dec.logits(), ref, 1e-4)
+    dec.close()
+    # f16 caches: the oracle's step on the f16 contents, this step's rows rounded before the attention reads them
+    kc16, vc16 = kc.astype(np.float16), vc.astype(np.float16)
+    dec = g.LlamaDecoder(gdev, kv_f16=True, **hp)
+    ref16 = _ref_step(w, hp, kc16.astype(np.float32), vc16.astype(np.float32), 31999, 2047, round_kv=True)
+    for fused in (3, 4):
+        _load(dec, w, kc16, vc16)
+        dec.decode(31999, 2047, fused)
+        _check(dec.logits(), ref16, 2e-4)
     dec.close()

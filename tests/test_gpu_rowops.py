@@ -75,10 +75,17 @@ def test_rope_vs_oracle(dev, t, h, hd, p0):
     pos = np.arange(p0, p0 + t, dtype=np.int32)
     ts = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
     got = _rope(dev, x, pos, 1.0, h, ts)
+    # The gate: the reference kernel's own f32 angle (rope.cu:16-20), rotation in f64.  What separates an f32 kernel
+    # from it is an ulp of powf times the angle (~1e-4 rad at position 2000) and f32 sin / cos: 3e-4 absolute on
+    # N(0,1) data.  A wrong exponent, pair index or position shows up at 1e-2 and more.
+    ref32 = npref.rope_f32_angles(x, pos, 1.0, h, ts)
+    err32 = np.max(np.abs(got.astype(np.float64) - ref32))
+    assert err32 < 3e-4, err32
+    # For information: against the oracle's f64 angle the rounding of the f32 angle itself (6e-8 relative of up to
+    # 2500 rad) is included as well.
     ref = oracle.rope(x, pos, 1.0, h, ts)
-    # f32 angle: theta up to ~2500 rad carries ~1e-7 relative error -> a few 1e-4 rad
     err = np.max(np.abs(got.astype(np.float64) - ref))
-    print("rope t=%d max abs err %.3g" % (t, err))
+    print("rope t=%d max abs err vs f32-angle reference %.3g, vs f64-angle oracle %.3g" % (t, err32, err))
     assert err < 2e-3 * max(1.0, (p0 + t) / 512.0)
     # pair norms are preserved to f32 rounding
     n0 = x[:, 0::2].astype(np.float64) ** 2 + x[:, 1::2].astype(np.float64) ** 2

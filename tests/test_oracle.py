@@ -316,3 +316,17 @@ def test_cpy_and_get_rows():
     w = oracle.quantize_q4_0((rng.standard_normal((10, 64)) * 0.02).astype(np.float32))
     ids = np.array([7, 0, 7, 9], np.int32)
     assert np.array_equal(oracle.get_rows_q4_0(w, ids), npref.q4_0_dequant(w)[ids])
+
+
+def test_rope_f32_angle_restatement_agrees_with_the_oracle():
+    """npref.rope_f32_angles (the reference kernel's f32 angle) against the oracle's f64 angle: identical where the
+    angle is exact in f32 (position 0, pair 0), and apart only by the rounding of the angle elsewhere."""
+    rng = np.random.default_rng(12)
+    h, hd = 4, 128
+    ts = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    for p0, tol in ((0, 2e-6), (100, 3e-5), (2040, 6e-4)):
+        pos = np.arange(p0, p0 + 5, dtype=np.int32)
+        x = rng.standard_normal((5 * h, hd)).astype(np.float32)
+        a, b = npref.rope_f32_angles(x, pos, 1.0, h, ts), oracle.rope(x, pos, 1.0, h, ts)
+        assert np.max(np.abs(a - b)) < tol, (p0, np.max(np.abs(a - b)))
+        assert np.max(np.abs(a[:, :2] - b[:, :2])) < 2e-6      # pair 0: theta = pos exactly
