@@ -102,34 +102,63 @@ def timed_graph(dev, fn, iters, reps=5):
     return float(np.median(out))
 
 
+def _host_cpus():
+    try:
+        return len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        return os.cpu_count() or 1
+
+
+def _time_cpu(fn, budget_s, max_passes=20000):
+    """One untimed pass, then whole passes until the budget is used: (passes, seconds)."""
+    fn()
+    t0 = time.perf_counter()
+    passes = 0
+    while True:
+        fn()
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or passes >= max_passes:
+            return passes, dt
+
+
 def cpu_baseline(weights_host, xs_host, budget_s):
     """The reference CPU op restated in C (oracle/), timed on this host.  4 threads is what the
     reference uses (nth = 4, src/op.rs:1438); the all-core figure is reported beside it."""
     import oracle  # the CPU leg is the only place the benchmark touches the oracle
-    ncpu = os.cpu_count() or 1
-    try:
-        ncpu = len(os.sched_getaffinity(0))
-    except (AttributeError, OSError):
-        pass
+    ncpu = _host_cpus()
     res = {}
     total = sum(w.nbytes for w in weights_host)
-    for label, nth in (("ref4", 4), ("all", max(1, min(ncpu, 64)))):
-        # one untimed pass, then whole passes until the budget is used
+
+    def one_pass(nth):
         for (k, n), w in zip(GEMV_SHAPES, weights_host):
             oracle.cpu_mul_mat_q4_0_f32(w, xs_host[k], nth)
-        t0 = time.perf_counter()
-        passes = 0
-        while True:
-            for (k, n), w in zip(GEMV_SHAPES, weights_host):
-                oracle.cpu_mul_mat_q4_0_f32(w, xs_host[k], nth)
-            passes += 1
-            dt = time.perf_counter() - t0
-            if dt > budget_s or passes >= 20000:
-                break
+
+    for label, nth in (("ref4", 4), ("all", max(1, min(ncpu, 64)))):
+        passes, dt = _time_cpu(lambda: one_pass(nth), budget_s)
         res[label] = {"value": total * passes / dt / 1e9, "unit": "GB/s", "cores": nth, "kind": "port",
                       "sample": "%d passes over the 4-shape GEMV set (%.0f MB of Q4_0 weights per pass), %.1f s"
                                 % (passes, total / 1e6, dt)}
     return res, ncpu
+
+
+def cpu_baseline_other_configs(w_4096x4096, w_4096x11008, x_vec, x_prefill, budget_s):
+    """The same CPU op on BASELINE.json configs[0] (one 4096 x 4096 matvec) and configs[2] (the M = 512 prefill
+    matmul, src/op.rs:1383-1598 with M > 1), each at the reference's 4 threads and at all cores."""
+    import oracle
+    ncpu = _host_cpus()
+    out = {"single_matvec_4096x4096": {}, "prefill_512x4096x11008": {}}
+    m, k, n = PREFILL
+    for label, nth in (("ref4", 4), ("all", max(1, min(ncpu, 64)))):
+        passes, dt = _time_cpu(lambda: oracle.cpu_mul_mat_q4_0_f32(w_4096x4096, x_vec, nth), budget_s)
+        out["single_matvec_4096x4096"][label] = {
+            "value": round(w_4096x4096.nbytes * passes / dt / 1e9, 2), "unit": "GB/s", "cores": nth, "kind": "port",
+            "us_per_matvec": round(dt / passes * 1e6, 1), "sample": "%d matvecs, %.1f s" % (passes, dt)}
+        passes, dt = _time_cpu(lambda: oracle.cpu_mul_mat_q4_0_f32(w_4096x11008, x_prefill, nth), budget_s)
+        out["prefill_512x4096x11008"][label] = {
+            "value": round(2.0 * m * k * n * passes / dt / 1e12, 4), "unit": "TFLOP/s", "cores": nth, "kind": "port",
+            "ms_per_matmul": round(dt / passes * 1e3, 1), "sample": "%d matmuls of 512 x 4096 x 11008, %.1f s" % (passes, dt)}
+    return out
 
 
 def _normal_f32(seed, count, scale, threads=16):
@@ -405,6 +434,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(avg_bytes / avg_us / 1e3, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(avg_bytes / avg_us / 1e3 / HBM_PEAK_GBPS, 4),
                      "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, summarised in "
+                                       "profiles/gemv_q4_0_group__llama7b_gemv_set.md (a constant from that profile, "
+                                       "not measured in this run)",
                      "kernel": "gemv_q4_0_group", "bytes_per_launch": avg_bytes, "us_per_launch": round(avg_us, 3)},
     }
     if not args.no_decode:
@@ -415,6 +447,9 @@ def main():
         out["cpu_baseline"] = res["ref4"]
         extra["cpu_baseline_all_cores"] = res["all"]
         extra["host_cpus_visible"] = ncpu
+        x_prefill = np.random.default_rng(5).standard_normal((PREFILL[0], PREFILL[1]), dtype=np.float32)
+        extra["cpu_baseline_other_configs"] = cpu_baseline_other_configs(
+            weights_host[0], weights_host[1], xs_host[4096], x_prefill, max(1.0, args.cpu_seconds / 4))
     out["extra"] = extra
     dev.close()
     print(json.dumps(out))

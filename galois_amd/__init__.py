@@ -250,6 +250,10 @@ class Device:
                                                            _ptr(v_cache), _ptr(out), n_head, head_dim, n_past,
                                                            _ptr(pos), freq_scale, theta_scale, scale))
 
+    def mul_mat_f16_f32(self, a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2):
+        self._check(self._lib.galois_hip_mul_mat_f16_f32(self._ctx, _ptr(a), _ptr(b), _ptr(dst), K, N, M, ne02, ne12,
+                                                         a_s0, a_s1, a_s2))
+
     def mul_mat_f32(self, a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2):
         self._check(self._lib.galois_hip_mul_mat_f32(self._ctx, _ptr(a), _ptr(b), _ptr(dst), K, N, M, ne02, ne12,
                                                      a_s0, a_s1, a_s2))

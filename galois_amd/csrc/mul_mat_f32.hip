@@ -1,11 +1,13 @@
-// f32 x f32 batched matmul over strided views: the two products of a decode step's attention over
-// the KV cache (scores = K^T q, out = V p), which the reference routes to cuBLAS sgemm after a cont()
-// copy (src/cuda.rs:698-782) or leaves as todo!() (src/cuda.rs:994-1010).
+// f32 x f32 and f16 x f32 batched matmul over strided views: the two products of a decode step's attention
+// over the KV cache (scores = K^T q, out = V p), which the reference routes to cuBLAS -- sgemm after a cont()
+// copy for f32 (src/cuda.rs:698-782, todo!() at src/cuda.rs:867-879), gemm_ex for an f16 src0
+// (CudaMatMul::f_x_y_y, src/cuda.rs:881-992 -> cuda_op_mul_mat_cublas, src/cuda.rs:698-782).
 //
 //   dst[i2][m][n] = sum_k a[(i2 / r2) * a_s2 + n * a_s1 + k * a_s0] * b[(i2 * M + m) * K + k]
 //
-// Both products read the cache exactly once and are HBM-bound.  With M == 1 (decode) two streaming
-// kernels are used; other shapes take the generic kernels.
+// a is f32 or f16 (widened exactly), b and dst f32, sums in f32.  Both attention products read the cache exactly
+// once and are HBM-bound.  With M == 1 (decode) two streaming kernels are used; f16 weights with M > 1 go to
+// the matrix cores (mul_mat_f16.hip); other shapes take the generic kernels.
 #include "common.h"
 
 namespace {
@@ -29,21 +31,32 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// Element loads of the a operand: f32 as it is, f16 widened.
+typedef _Float16 mm_half4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float mm_ld1(const float *p) { return *p; }
+__device__ __forceinline__ float mm_ld1(const _Float16 *p) { return (float)*p; }
+__device__ __forceinline__ float4 mm_ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 mm_ld4(const _Float16 *p) {
+    const mm_half4 h = *reinterpret_cast<const mm_half4 *>(p);
+    return make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w);
+}
+
 // ---- generic kernels (any K, N, M) ---------------------------------------------------------------
 
 // Rows of `a` contiguous along K (a_s0 == 1).  One wave per (n, i2).
-__global__ __launch_bounds__(kThreads) void mul_mat_f32_krows(const float *__restrict__ a, const float *__restrict__ b,
+template <typename AT>
+__global__ __launch_bounds__(kThreads) void mul_mat_f32_krows(const AT *__restrict__ a, const float *__restrict__ b,
                                                               float *__restrict__ dst, int K, int N, int M, int r2,
                                                               int64_t a_s1, int64_t a_s2) {
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     const int i2 = blockIdx.y;
     if (n >= N) return;
-    const float *ar = a + (int64_t)(i2 / r2) * a_s2 + (int64_t)n * a_s1;
+    const AT *ar = a + (int64_t)(i2 / r2) * a_s2 + (int64_t)n * a_s1;
     for (int m = 0; m < M; m++) {
         const float *br = b + ((int64_t)i2 * M + m) * K;
         float acc = 0.0f;
-        for (int k = lane; k < K; k += 64) acc = __builtin_fmaf(ar[k], br[k], acc);
+        for (int k = lane; k < K; k += 64) acc = __builtin_fmaf(mm_ld1(ar + k), br[k], acc);
         acc = group_sum<64>(acc);
         if (lane == 0) dst[((int64_t)i2 * M + m) * N + n] = acc;
     }
@@ -51,19 +64,20 @@ __global__ __launch_bounds__(kThreads) void mul_mat_f32_krows(const float *__res
 
 // `a` contiguous along N (a_s1 == 1, K strided by a_s0).  A workgroup owns 64 columns n of one
 // batch slice; its 4 waves split K and combine through LDS.
-__global__ __launch_bounds__(kThreads) void mul_mat_f32_ncols(const float *__restrict__ a, const float *__restrict__ b,
+template <typename AT>
+__global__ __launch_bounds__(kThreads) void mul_mat_f32_ncols(const AT *__restrict__ a, const float *__restrict__ b,
                                                               float *__restrict__ dst, int K, int N, int M, int r2,
                                                               int64_t a_s0, int64_t a_s2) {
     __shared__ float part[kThreads];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + lane;
     const int i2 = blockIdx.y;
-    const float *ab = a + (int64_t)(i2 / r2) * a_s2;
+    const AT *ab = a + (int64_t)(i2 / r2) * a_s2;
     for (int m = 0; m < M; m++) {
         const float *br = b + ((int64_t)i2 * M + m) * K;
         float acc = 0.0f;
         if (n < N)
-            for (int k = wave; k < K; k += kThreads / 64) acc = __builtin_fmaf(ab[(int64_t)k * a_s0 + n], br[k], acc);
+            for (int k = wave; k < K; k += kThreads / 64) acc = __builtin_fmaf(mm_ld1(ab + (int64_t)k * a_s0 + n), br[k], acc);
         part[threadIdx.x] = acc;
         __syncthreads();
         if (wave == 0 && n < N)
@@ -78,8 +92,8 @@ __global__ __launch_bounds__(kThreads) void mul_mat_f32_ncols(const float *__res
 // wave-load covers 64 / LPR rows, and a wave keeps U wave-loads in flight before it reduces any.
 // Rows are numbered with the batch index fastest when that is the smaller stride, so that the rows
 // of one wave-load (and of neighbouring waves) are neighbours in memory.
-template <int LPR, int U>
-__global__ __launch_bounds__(kThreads) void mul_vec_f32_krows(const float *__restrict__ a, const float *__restrict__ b,
+template <int LPR, int U, typename AT>
+__global__ __launch_bounds__(kThreads) void mul_vec_f32_krows(const AT *__restrict__ a, const float *__restrict__ b,
                                                               float *__restrict__ dst, int N, int ne12, int r2,
                                                               int64_t a_s1, int64_t a_s2, int batch_fastest) {
     constexpr int RPL = 64 / LPR, K = LPR * 4;
@@ -96,7 +110,7 @@ __global__ __launch_bounds__(kThreads) void mul_vec_f32_krows(const float *__res
         const int64_t rc = r < R ? r : R - 1;
         const int64_t i2 = batch_fastest ? rc % ne12 : rc / N;
         const int64_t n = batch_fastest ? rc / ne12 : rc % N;
-        av[u] = *reinterpret_cast<const float4 *>(a + (i2 / r2) * a_s2 + n * a_s1 + kl * 4);
+        av[u] = mm_ld4(a + (i2 / r2) * a_s2 + n * a_s1 + kl * 4);
         bv[u] = *reinterpret_cast<const float4 *>(b + i2 * K + kl * 4);
         out[u] = r < R ? i2 * N + n : -1;
     }
@@ -117,7 +131,8 @@ __global__ __launch_bounds__(kThreads) void mul_vec_f32_krows(const float *__res
 // With more than one slab the workgroup writes its partial sums to `part` and sum_slabs_f32 adds the
 // slabs in slab order afterwards, so the result is the same on every launch.
 constexpr int kVecRows = 16;
-__global__ __launch_bounds__(kThreads) void mul_vec_f32_ncols(const float *__restrict__ a, const float *__restrict__ b,
+template <typename AT>
+__global__ __launch_bounds__(kThreads) void mul_vec_f32_ncols(const AT *__restrict__ a, const float *__restrict__ b,
                                                               float *__restrict__ dst, float *__restrict__ part, int K, int N, int C, int r2,
                                                               int64_t a_s0, int64_t a_s2, int rows_per_wave) {
     __shared__ float4 red[kThreads / 64][64];
@@ -127,7 +142,7 @@ __global__ __launch_bounds__(kThreads) void mul_vec_f32_ncols(const float *__res
     const bool col_ok = c < C;  // C and N are multiples of 4: a lane's four columns stay in one batch slice
     const int cc = col_ok ? c : 0;
     const int i2 = cc / N, n = cc % N;
-    const float *ac = a + (int64_t)(i2 / r2) * a_s2 + n;
+    const AT *ac = a + (int64_t)(i2 / r2) * a_s2 + n;
     const float *bc = b + (int64_t)i2 * K;
     const int k_begin = (slab * (kThreads / 64) + wave) * rows_per_wave;
     const int k_end = min(K, k_begin + rows_per_wave);
@@ -139,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void mul_vec_f32_ncols(const float *__res
         for (int u = 0; u < kVecRows; u++) {
             const int k = k0 + u;
             const int kc = k < k_end ? k : k_end - 1;
-            v[u] = *reinterpret_cast<const float4 *>(ac + (int64_t)kc * a_s0);
+            v[u] = mm_ld4(ac + (int64_t)kc * a_s0);
             p[u] = bc[kc];
         }
 #pragma unroll
@@ -182,30 +197,42 @@ __global__ __launch_bounds__(kThreads) void sum_slabs_f32(const float *__restric
     dst[c] = s;
 }
 
-template <int LPR>
-void launch_vec_krows(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int N, int ne12, int r2,
+template <int LPR, typename AT>
+void launch_vec_krows(galois_hip_ctx *ctx, const AT *a, const float *b, float *dst, int N, int ne12, int r2,
                       int64_t a_s1, int64_t a_s2) {
     constexpr int U = 8, rows_per_wg = (kThreads / 64) * (64 / LPR) * U;
     const int64_t R = (int64_t)N * ne12;
-    hipLaunchKernelGGL((mul_vec_f32_krows<LPR, U>), dim3((unsigned)((R + rows_per_wg - 1) / rows_per_wg)),
+    hipLaunchKernelGGL((mul_vec_f32_krows<LPR, U, AT>), dim3((unsigned)((R + rows_per_wg - 1) / rows_per_wg)),
                        dim3(kThreads), 0, ctx->stream, a, b, dst, N, ne12, r2, a_s1, a_s2, (int)(a_s2 < a_s1));
 }
 
 }  // namespace
 
-extern "C" int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K,
-                                          int32_t N, int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1,
-                                          int64_t a_s2) {
+// gemm_f16_f32_mfma (mul_mat_f16.hip): f16 rows contiguous along K against M > 1 rows of b on the matrix cores;
+// returns false when the operands do not fit it (the generic kernels then serve the call).
+bool gh_mul_mat_f16_mfma(galois_hip_ctx *ctx, const _Float16 *a, const float *b, float *dst, int K, int N, int M,
+                         int ne02, int ne12, int64_t a_s1, int64_t a_s2);
+
+namespace {
+
+template <typename AT>
+int32_t mul_mat_any(galois_hip_ctx *ctx, const AT *a, const float *b, float *dst, int32_t K, int32_t N, int32_t M,
+                    int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2) {
+    constexpr bool F16 = sizeof(AT) == 2;
+    constexpr size_t A16 = F16 ? 8 : 16;  // alignment of a four-element load
     GH_REQUIRE_CTX(ctx);
     GH_REQUIRE(ctx, a && b && dst, GALOIS_HIP_E_NULL, "mul_mat_f32");
     GH_REQUIRE(ctx, K > 0 && N > 0 && M > 0 && ne02 > 0 && ne12 > 0 && ne12 % ne02 == 0 && ne12 <= 65535,
                GALOIS_HIP_E_SHAPE, "mul_mat_f32");
     GH_REQUIRE(ctx, a_s0 == 1 || a_s1 == 1, GALOIS_HIP_E_UNSUPPORTED,
                "mul_mat_f32: a must be contiguous along K (a_s0 == 1) or along N (a_s1 == 1)");
-    GH_REQUIRE(ctx, gh_aligned(a, 4) && gh_aligned(b, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "mul_mat_f32");
+    GH_REQUIRE(ctx, gh_aligned(a, sizeof(AT)) && gh_aligned(b, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN, "mul_mat_f32");
     GH_BIND(ctx);
     const int r2 = ne12 / ne02;
-    const bool vec16 = M == 1 && gh_aligned(a, 16) && gh_aligned(b, 16) && a_s2 % 4 == 0;
+    if (F16 && M > 1 && a_s0 == 1 &&
+        gh_mul_mat_f16_mfma(ctx, (const _Float16 *)a, b, dst, K, N, M, ne02, ne12, a_s1, a_s2))
+        GH_LAUNCH_CHECK(ctx, "mul_mat_f16_f32 launch");
+    const bool vec16 = M == 1 && gh_aligned(a, A16) && gh_aligned(b, 16) && a_s2 % 4 == 0;
     if (a_s0 == 1) {
         const bool fast = vec16 && a_s1 % 4 == 0 && (K == 32 || K == 64 || K == 128 || K == 256);
         if (fast) {
@@ -216,7 +243,7 @@ extern "C" int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, c
                 default: launch_vec_krows<64>(ctx, a, b, dst, N, ne12, r2, a_s1, a_s2); break;
             }
         } else {
-            hipLaunchKernelGGL(mul_mat_f32_krows, dim3((N + 3) / 4, ne12), dim3(kThreads), 0, ctx->stream, a, b, dst, K,
+            hipLaunchKernelGGL(mul_mat_f32_krows<AT>, dim3((N + 3) / 4, ne12), dim3(kThreads), 0, ctx->stream, a, b, dst, K,
                                N, M, r2, a_s1, a_s2);
         }
     } else {
@@ -231,15 +258,29 @@ extern "C" int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, c
                           (nslabs == 1 || (int64_t)nslabs * C <= GH_PARTIAL_FLOATS) && ctx->scratch != nullptr;
         if (fast) {
             float *part = (float *)ctx->scratch;
-            hipLaunchKernelGGL(mul_vec_f32_ncols, dim3((unsigned)tiles, nslabs), dim3(kThreads), 0, ctx->stream, a, b,
+            hipLaunchKernelGGL(mul_vec_f32_ncols<AT>, dim3((unsigned)tiles, nslabs), dim3(kThreads), 0, ctx->stream, a, b,
                                dst, part, K, N, (int)C, r2, a_s0, a_s2, rows_per_wave);
             if (nslabs > 1)
                 hipLaunchKernelGGL(sum_slabs_f32, dim3((unsigned)((C + kThreads - 1) / kThreads)), dim3(kThreads), 0,
                                    ctx->stream, part, dst, (int)C, nslabs);
         } else {
-            hipLaunchKernelGGL(mul_mat_f32_ncols, dim3((N + 63) / 64, ne12), dim3(kThreads), 0, ctx->stream, a, b, dst,
+            hipLaunchKernelGGL(mul_mat_f32_ncols<AT>, dim3((N + 63) / 64, ne12), dim3(kThreads), 0, ctx->stream, a, b, dst,
                                K, N, M, r2, a_s0, a_s2);
         }
     }
     GH_LAUNCH_CHECK(ctx, "mul_mat_f32 launch");
+}
+
+}  // namespace
+
+extern "C" int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K,
+                                          int32_t N, int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1,
+                                          int64_t a_s2) {
+    return mul_mat_any<float>(ctx, a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2);
+}
+
+extern "C" int32_t galois_hip_mul_mat_f16_f32(galois_hip_ctx *ctx, const void *a, const float *b, float *dst, int32_t K,
+                                              int32_t N, int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0,
+                                              int64_t a_s1, int64_t a_s2) {
+    return mul_mat_any<_Float16>(ctx, (const _Float16 *)a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2);
 }

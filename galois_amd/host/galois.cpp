@@ -177,6 +177,7 @@ static bool all_gpu(std::initializer_list<const Tensor *> ts, std::shared_ptr<Cu
 // f32 x f32 arm (the products over the KV cache).  The reference routes this case to a todo!()
 // (src/cuda.rs:994-1010) after a cuBLAS sgemm path for F16 weights (:698-782); here src0 may be
 // any strided 3-D view, so a permuted cache needs no cont() copy first.
+// (F32 | F16, F32) -> F32 over strided views of src0.
 static GResult matmul_f32(const CudaDevice &dev, const Tensor &a, const Tensor &b, Tensor &dst) {
     const Dim &ad = a.dim(), &bd = b.dim(), &dd = dst.dim();
     if (ad.shape[0] != bd.shape[0]) return err(GError::ShapeError, "matmul: ne00 != ne10");
@@ -186,10 +187,13 @@ static GResult matmul_f32(const CudaDevice &dev, const Tensor &a, const Tensor &
     if (ad.shape[2] == 0 || bd.shape[2] % ad.shape[2] != 0) return err(GError::ShapeError, "matmul: src0 must broadcast over ne12");
     if (!bd.ggml_is_contiguous(b.dtype()) || !dd.ggml_is_contiguous(dst.dtype()))
         return err(GError::Unimplemented, "matmul f32: src1 and dst must be contiguous");
-    return dev.check(galois_hip_mul_mat_f32(dev.ctx(), (const float *)a.data(), (const float *)b.data(), (float *)dst.data(),
-                                            (int32_t)ad.shape[0], (int32_t)ad.shape[1], (int32_t)bd.shape[1],
-                                            (int32_t)ad.shape[2], (int32_t)bd.shape[2], (int64_t)ad.stride[0],
-                                            (int64_t)ad.stride[1], (int64_t)ad.stride[2]));
+    // an F16 src0 is the (F16, F32) -> F32 arm that the reference hands to cuBLAS (CudaMatMul::f_x_y_y,
+    // src/cuda.rs:881-992): the same views, the a operand widened exactly
+    auto fn = a.dtype() == GGmlType::F16 ? (decltype(&galois_hip_mul_mat_f16_f32))galois_hip_mul_mat_f16_f32
+                                         : (decltype(&galois_hip_mul_mat_f16_f32))galois_hip_mul_mat_f32;
+    return dev.check(fn(dev.ctx(), a.data(), (const float *)b.data(), (float *)dst.data(), (int32_t)ad.shape[0],
+                        (int32_t)ad.shape[1], (int32_t)bd.shape[1], (int32_t)ad.shape[2], (int32_t)bd.shape[2],
+                        (int64_t)ad.stride[0], (int64_t)ad.stride[1], (int64_t)ad.stride[2]));
 }
 
 // galois_matmul, src/op.rs:3093-3111 -> CudaMatMul.map -> f_q_f32_f32 (src/cuda.rs:994-1139).
@@ -197,10 +201,10 @@ GResult galois_matmul(const Tensor &a, const Tensor &b, Tensor &dst) {
     std::shared_ptr<CudaDevice> dev;
     if (!all_gpu({&a, &b, &dst}, &dev))
         return err(GError::Unimplemented, "galois_matmul: only (Gpu, Gpu, Gpu) operands on one device (the reference's other arms are todo!() or CPU)");
-    if (a.dtype() == GGmlType::F32 && b.dtype() == GGmlType::F32 && dst.dtype() == GGmlType::F32)
+    if ((a.dtype() == GGmlType::F32 || a.dtype() == GGmlType::F16) && b.dtype() == GGmlType::F32 && dst.dtype() == GGmlType::F32)
         return matmul_f32(*dev, a, b, dst);
     if (!(a.dtype() == GGmlType::Q4_0 && b.dtype() == GGmlType::F32 && dst.dtype() == GGmlType::F32))
-        return err(GError::Unimplemented, "galois_matmul: only (Q4_0 | F32, F32) -> F32 (CudaMap2::map, src/cuda.rs:476-521)");
+        return err(GError::Unimplemented, "galois_matmul: only (Q4_0 | F16 | F32, F32) -> F32 (CudaMap2::map, src/cuda.rs:476-521)");
     const Dim &ad = a.dim(), &bd = b.dim(), &dd = dst.dim();
     const size_t ne00 = ad.shape[0], ne01 = ad.shape[1], ne02 = ad.shape[2], ne03 = ad.shape[3];
     const size_t ne10 = bd.shape[0], ne11 = bd.shape[1], ne12 = bd.shape[2], ne13 = bd.shape[3];

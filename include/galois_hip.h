@@ -227,6 +227,14 @@ int32_t galois_hip_get_rows_q4_0(galois_hip_ctx *ctx, const void *table, const i
 int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float *b, float *dst, int32_t K, int32_t N,
                                int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2);
 
+/* The same with an f16 a (element strides count halfs): the (F16, F32) -> F32 arm of galois_matmul, which the
+ * reference serves with cuBLAS gemm_ex on f16 operands with f16 accumulation and an f16 result
+ * (CudaMatMul::f_x_y_y, src/cuda.rs:881-992 -> cuda_op_mul_mat_cublas, src/cuda.rs:698-757).  Here a is widened
+ * exactly and sums are f32; with M > 1 and rows of a contiguous along K (K % 32 == 0, 16-byte aligned rows) the
+ * product runs on the matrix cores with b rounded to f16 as the reference's convert_fp32_to_fp16 does. */
+int32_t galois_hip_mul_mat_f16_f32(galois_hip_ctx *ctx, const void *a, const float *b, float *dst, int32_t K, int32_t N,
+                                   int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2);
+
 /* Attention of one decode step over an f32 KV cache in two launches instead of the nine of the op sequence
  * rope_custom(q), rope_custom(k), cpy(k -> cache), cpy(v -> cache), matmul(K^T, q), scale, soft_max, matmul(V, p)
  * (src/cuda.rs:1257-1356, 1382-1595, 698-782, 1597-1663), with the same arithmetic up to the order of f32 sums:
