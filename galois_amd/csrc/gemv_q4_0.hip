@@ -143,22 +143,6 @@ __device__ __forceinline__ void fetch_task(const float *xs /* the slot's 64 acti
 // nibble order of the weight dword: byte b low, byte b high, byte b+1 low, byte b+1 high, ...
 #define GH_TASK_X8(v) {(v)[0].x, (v)[1].x, (v)[0].y, (v)[1].y, (v)[2].x, (v)[3].x, (v)[2].y, (v)[3].y}
 
-// What a lane reads of its slot before the dot products.
-template <int L>
-__device__ __forceinline__ uint32_t read_slot_planes(const uint32_t *src, uint32_t (&xl)[L][8], float &sA, float &sB) {
-#pragma unroll
-    for (int l = 0; l < L; l++) {
-        const uint4 a = *reinterpret_cast<const uint4 *>(src + l * 8);
-        const uint4 b = *reinterpret_cast<const uint4 *>(src + l * 8 + 4);
-        xl[l][0] = a.x, xl[l][1] = a.y, xl[l][2] = a.z, xl[l][3] = a.w;
-        xl[l][4] = b.x, xl[l][5] = b.y, xl[l][6] = b.z, xl[l][7] = b.w;
-    }
-    const uint4 sc = *reinterpret_cast<const uint4 *>(src + 8 * L);
-    sA = __builtin_bit_cast(float, sc.x);
-    sB = __builtin_bit_cast(float, sc.y);
-    return sc.z | sc.w;  // non-zero: a block of the slot has a correction
-}
-
 // Activation preparation, split in two so that the activation loads can be issued before
 // the first weight loads (loads return in order, so whatever must be consumed first has to
 // be requested first) and the arithmetic runs while the weights are in flight.
@@ -202,58 +186,72 @@ __device__ __forceinline__ int sdot8_first(uint32_t a, uint32_t b) {
     return d;
 }
 
-// Integer dot of one block's four nibble dwords with its L planes: sum_l 16^l * dot8.
-// One accumulator per plane, issued round-robin: back-to-back v_dot8 into the same
+// Integer dot of one block's four nibble dwords with the block's four dwords of each of its L planes:
+// sum_l 16^l * dot8.  One accumulator per plane, issued round-robin: back-to-back v_dot8 into the same
 // register serialise on the dot pipeline's latency, independent ones issue every cycle.
 template <int L>
-__device__ __forceinline__ int block_dot(const uint32_t nd[4], const uint32_t (&xl)[L][8], int base) {
+__device__ __forceinline__ int block_dot(const uint32_t (&nd)[4], const uint32_t (&xh)[L][4]) {
     int t[L];
 #pragma unroll
-    for (int l = 0; l < L; l++) t[l] = sdot8_first(nd[0], xl[l][base]);
+    for (int l = 0; l < L; l++) t[l] = sdot8_first(nd[0], xh[l][0]);
 #pragma unroll
     for (int i = 1; i < 4; i++)
 #pragma unroll
-        for (int l = 0; l < L; l++) t[l] = __builtin_amdgcn_sdot8((int)nd[i], (int)xl[l][base + i], t[l], false);
+        for (int l = 0; l < L; l++) t[l] = __builtin_amdgcn_sdot8((int)nd[i], (int)xh[l][i], t[l], false);
     int r = t[L - 1];
 #pragma unroll
     for (int l = L - 2; l >= 0; l--) r = (r << 4) + t[l];
     return r;
 }
 
-template <int L>
-__device__ __forceinline__ float slot_dot(const q4_slot &q, const uint32_t (&xl)[L][8], float sA, float sB) {
-    const float dA = f16_bits_to_f32(q.w[0] & 0xFFFFu);
-    const float dB = f16_bits_to_f32(q.w[4] >> 16);
-    const uint32_t sign = 0x88888888u;
-    // block A's qs start 2 bytes into the slot: each of its dwords is the top half of one word and the low half of the next
-    const uint32_t ndA[4] = {__builtin_amdgcn_alignbit(q.w[1], q.w[0], 16) ^ sign, __builtin_amdgcn_alignbit(q.w[2], q.w[1], 16) ^ sign,
-                             __builtin_amdgcn_alignbit(q.w[3], q.w[2], 16) ^ sign, __builtin_amdgcn_alignbit(q.w[4], q.w[3], 16) ^ sign};
-    const uint32_t ndB[4] = {q.w[5] ^ sign, q.w[6] ^ sign, q.w[7] ^ sign, q.w[8] ^ sign};
-    const int tA = block_dot<L>(ndA, xl, 0);
-    const int tB = block_dot<L>(ndB, xl, 4);
-    float r = (dA * sA) * (float)tA;
-    r = __builtin_fmaf(dB * sB, (float)tB, r);
-    return r;
-}
-
-// The correction of one slot for one row: the slot's weights once more (they are in the caches: the row was just
-// read) against the correction planes of the slot's residuals.
-template <int L>
-__device__ __forceinline__ float slot_correction(const uint8_t *w_slot, const uint32_t *slot_src, const uint32_t *corr_src) {
+// One slot of R rows: acc[r] += the dot product of row r's 64 weights (q[r]) with the slot's activations, read from
+// the slot's LDS image (slot_lds) one block at a time, so that only half a slot's planes are held at once; a block
+// with a correction (few, if any) also takes the same weights against its correction planes.
+template <int L, int R>
+__device__ __forceinline__ void slot_rows(const q4_slot (&q)[R], const uint32_t *slot_src, const uint32_t *corr_src,
+                                          float *acc /* [R] */) {
     constexpr int CL = xprep::CORR_L;
-    uint32_t xc[CL][8];
+    const uint32_t sign = 0x88888888u;
+    const uint4 sc = *reinterpret_cast<const uint4 *>(slot_src + 8 * L);  // scales of A, B; of their corrections (0 = none)
 #pragma unroll
-    for (int l = 0; l < CL; l++) {
-        const uint4 a = *reinterpret_cast<const uint4 *>(corr_src + l * 8);
-        const uint4 b = *reinterpret_cast<const uint4 *>(corr_src + l * 8 + 4);
-        xc[l][0] = a.x, xc[l][1] = a.y, xc[l][2] = a.z, xc[l][3] = a.w;
-        xc[l][4] = b.x, xc[l][5] = b.y, xc[l][6] = b.z, xc[l][7] = b.w;
+    for (int blk = 0; blk < 2; blk++) {
+        uint32_t xh[L][4];
+#pragma unroll
+        for (int l = 0; l < L; l++) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(slot_src + l * 8 + 4 * blk);
+            xh[l][0] = v.x, xh[l][1] = v.y, xh[l][2] = v.z, xh[l][3] = v.w;
+        }
+        const float s = __builtin_bit_cast(float, blk ? sc.y : sc.x);
+        const uint32_t cbits = blk ? sc.w : sc.z;
+        uint32_t nd[R][4];
+        float d[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (blk == 0) {
+                // block A's qs start 2 bytes into the slot: each of its dwords is the top half of one word and the
+                // low half of the next
+                d[r] = f16_bits_to_f32(q[r].w[0] & 0xFFFFu);
+#pragma unroll
+                for (int i = 0; i < 4; i++) nd[r][i] = __builtin_amdgcn_alignbit(q[r].w[i + 1], q[r].w[i], 16) ^ sign;
+            } else {
+                d[r] = f16_bits_to_f32(q[r].w[4] >> 16);
+#pragma unroll
+                for (int i = 0; i < 4; i++) nd[r][i] = q[r].w[5 + i] ^ sign;
+            }
+            acc[r] = __builtin_fmaf(d[r] * s, (float)block_dot<L>(nd[r], xh), acc[r]);
+        }
+        if (cbits != 0) {
+            uint32_t xc[CL][4];
+#pragma unroll
+            for (int l = 0; l < CL; l++) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(corr_src + l * 8 + 4 * blk);
+                xc[l][0] = v.x, xc[l][1] = v.y, xc[l][2] = v.z, xc[l][3] = v.w;
+            }
+            const float s2 = __builtin_bit_cast(float, cbits);
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] = __builtin_fmaf(d[r] * s2, (float)block_dot<CL>(nd[r], xc), acc[r]);
+        }
     }
-    const uint2 sc = *reinterpret_cast<const uint2 *>(slot_src + 8 * L + 2);
-    // a block without a correction has scale 0 and planes nobody wrote: whatever integer they give is multiplied by 0
-    q4_slot q;
-    load_slot(q, w_slot);
-    return slot_dot<CL>(q, xc, __builtin_bit_cast(float, sc.x), __builtin_bit_cast(float, sc.y));
 }
 
 // Fast path: K % 64 == 0, W 4-byte aligned, x 8-byte aligned.
@@ -299,15 +297,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
         xp.compute(lds, xg, c0, cs);
         __syncthreads();
 
-        uint32_t cmask = 0;  // bit i: this lane's slot of step i has a correction
-        int step = 0;
-        for (int sl = lane; sl - lane < cs; sl += 64, step++) {  // uniform trip count; lanes past the end idle
+        const uint32_t *corr = lds + cs * SD;
+        for (int sl = lane; sl - lane < cs; sl += 64) {  // uniform trip count; lanes past the end idle
             const bool act = sl < cs;
             const int s_ld = min(sl, cs - 1);
-            uint32_t xl[L][8];
-            float sA, sB;
-            const uint32_t has_corr = read_slot_planes<L>(lds + s_ld * SD, xl, sA, sB);
-            if (act && has_corr) cmask |= 1u << step;
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 q4_slot q[R];
@@ -320,25 +313,8 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_dot8(const uint8_t 
                         load_slot(q[r], W + (size_t)min(row0 + g * R + r, N - 1) * row_bytes +
                                             (size_t)(c0 + s_ld) * sizeof(q4_slot));
                 }
-                if (act) {
-#pragma unroll
-                    for (int r = 0; r < R; r++) acc[g][r] += slot_dot<L>(q[r], xl, sA, sB);
-                }
+                if (act) slot_rows<L, R>(q, lds + s_ld * SD, corr + s_ld * slot_lds<L>::corr_dwords, acc[g]);
             }
-        }
-        if (cmask) {  // rare: only lanes whose slots have corrections get here
-            const uint32_t *corr = lds + cs * SD;
-            for (int st = 0; st < (kChunkSlots + 63) / 64; st++)
-                if (cmask >> st & 1) {
-                    const int s = st * 64 + lane;
-#pragma unroll
-                    for (int g = 0; g < G; g++)
-#pragma unroll
-                        for (int r = 0; r < R; r++)
-                            acc[g][r] += slot_correction<L>(W + (size_t)min(row0 + g * R + r, N - 1) * row_bytes +
-                                                                (size_t)(c0 + s) * sizeof(q4_slot),
-                                                            lds + s * SD, corr + s * slot_lds<L>::corr_dwords);
-                }
         }
     }
 
@@ -656,15 +632,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
 
     // The rows of this wave.  The first slots are the ones requested before the preparation.
     {
-        uint32_t cmask = 0;  // bit i: this lane's slot of step i has a correction
-        int step = 0;
-        for (int sl = lane; sl - lane < ns; sl += 64, step++) {  // uniform trip count; lanes past the end idle
+        const uint32_t *corr = lds + ns * SD + ((NORM && PG == 1) ? ns * 64 : 0);
+        for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
             const bool act = sl < ns;
             const int s_ld = min(sl, ns - 1);
-            uint32_t xl[L][8];
-            float sA, sB;
-            const uint32_t has_corr = read_slot_planes<L>(lds + s_ld * SD, xl, sA, sB);
-            if (act && has_corr) cmask |= 1u << step;
             q4_slot q[R];
             if (sl == lane) {
 #pragma unroll
@@ -677,24 +648,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
                     load_slot(q[j], base + (size_t)row * row_bytes + (size_t)s_ld * sizeof(q4_slot));
                 }
             }
-            if (act) {
-#pragma unroll
-                for (int j = 0; j < R; j++) acc[j] += slot_dot<L>(q[j], xl, sA, sB);
-            }
-        }
-        if (cmask) {  // rare: only lanes whose slots have corrections get here
-            const uint32_t *corr = lds + ns * SD + ((NORM && PG == 1) ? ns * 64 : 0);
-            for (int st = 0; st < (GG_MAX_SLOTS + 63) / 64; st++)
-                if (cmask >> st & 1) {
-                    const int s = st * 64 + lane;
-#pragma unroll
-                    for (int j = 0; j < R; j++) {
-                        const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
-                        const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
-                        acc[j] += slot_correction<L>(base + (size_t)row * row_bytes + (size_t)s * sizeof(q4_slot),
-                                                     lds + s * SD, corr + s * slot_lds<L>::corr_dwords);
-                    }
-                }
+            if (act) slot_rows<L, R>(q, lds + s_ld * SD, corr + s_ld * slot_lds<L>::corr_dwords, acc);
         }
 
         // every total lands in lane 63; lane j picks up row j so the wave stores its rows at once

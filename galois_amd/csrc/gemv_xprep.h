@@ -13,11 +13,15 @@
 // What the rounding drops is not lost.  The residual r = x - X * 2^(e-XBITS+1) is exact in f32 and at most half a
 // grid step, 2^(e-XBITS).  That is 2^(1-XBITS) of a block's largest activation, but it can be all of a small one:
 // a block in which one activation towers over the rest leaves the rest few bits, or none.  The decision is made on
-// the sum of |x| over the block without its largest activation: if that sum is below 31 half steps times 2^14, the
+// the sum of |x| over the block without its largest activation: if that sum is below 31 half steps times 2^13, the
 // block gets a correction block -- the residuals of its activations below the top binade, in the same fixed-point
 // form with their own scale and CORR_L limbs -- and the kernel adds dot(weights, correction planes) for it, which
 // takes those activations to 2^-13 of their largest residual (at most 2^-31 of the block's largest activation).
-// In every other block the activations other than the largest satisfy  sum |r_k| <= 2^-14 * sum |x_k|.
+// In every other block the activations other than the largest satisfy  sum |r_k| <= 2^-13 * sum |x_k|
+// (the bound; rounding errors are spread over +-half a step, so the typical sum is half of that and signed).
+// The threshold is a trade: a block of 32 N(0,1) values is never flagged, the product-shaped values of a SwiGLU
+// (silu(g) * u) once in two thousand blocks; at 2^14 it was one block in fifty, enough for every workgroup of a
+// down projection to run the correction code for a lane or two in every pass.
 // A block too small for a grid of its own (largest activation below 2^-108) lives in its correction block alone.
 //
 // Plain C++ (no HIP builtins) so the same code is unit-tested on the CPU.
@@ -98,7 +102,7 @@ GH_HD float residual(float x, float mult, float scale) {
 }
 
 constexpr int CORR_L = 4;                       // limbs of a correction block
-constexpr float CORR_REST_FACTOR = 253952.0f;   // 31 * 2^13: 31 half grid steps times 2^14, in grid steps
+constexpr float CORR_REST_FACTOR = 126976.0f;   // 31 * 2^12: 31 half grid steps times 2^13, in grid steps
 
 // Whether |x| (as f32 bits with the sign cleared) lies below the top binade of a block whose largest |x| has the
 // bits amax_bits: a correction block holds the residuals of such activations only (the others keep 2^(1-XBITS)).

@@ -223,7 +223,28 @@ GResult galois_matmul(const Tensor &a, const Tensor &b, Tensor &dst) {
     const uint8_t *w = (const uint8_t *)a.data();
     const float *x = (const float *)b.data();
     float *y = (float *)dst.data();
-    for (size_t i0 = 0; i0 < ne13 * ne12; i0++) {  // src/cuda.rs:1026-1034 and :1076-1134
+    // Batch slices of a decode product (ne11 == 1): the reference launches one kernel per slice (the loop at
+    // src/cuda.rs:1026-1034); here up to eight slices go out per launch when the grouped kernel takes the shape
+    // (a launch gap costs as much as streaming ~15 MB of weights).  Same results bit for bit.
+    const size_t nslices = ne13 * ne12;
+    if (ne11 == 1 && nslices > 1 && ne00 % 64 == 0 && ne00 <= 12288 && ((uintptr_t)w % 4) == 0 && ((uintptr_t)x % 8) == 0 &&
+        (ne01 * (ne00 / 32) * 18) % 4 == 0 && (ne10 * sizeof(float)) % 8 == 0) {
+        for (size_t i0 = 0; i0 < nslices; i0 += 8) {
+            galois_hip_gemv_item items[8];
+            const size_t n = nslices - i0 < 8 ? nslices - i0 : 8;
+            memset(items, 0, sizeof(items));
+            for (size_t j = 0; j < n; j++) {
+                items[j].vx = w + ((i0 + j) / i02_divisor) * ne01 * (ne00 / 32) * 18;
+                items[j].y = x + (i0 + j) * ne10;
+                items[j].dst = y + (i0 + j) * ne0;
+                items[j].ncols = (int32_t)ne00, items[j].nrows = (int32_t)ne01;
+            }
+            GResult r = dev->check(galois_hip_dequantize_mul_mat_vec_q4_0_group(dev->ctx(), items, (int32_t)n));
+            if (!r.ok()) return r;
+        }
+        return ok();
+    }
+    for (size_t i0 = 0; i0 < nslices; i0++) {  // src/cuda.rs:1026-1034 and :1076-1134
         const uint8_t *wi = w + (i0 / i02_divisor) * ne01 * (ne00 / 32) * 18;
         const float *xi = x + i0 * ne11 * ne10;
         float *yi = y + i0 * ne1 * ne0;

@@ -32,21 +32,22 @@ def test_cuda_matmul_gemv_and_prefill(gpu):
         assert emax < tol and el2 < tol, (m, emax, el2)
 
 
-def test_cuda_matmul_batched_broadcast(gpu):
-    """src0 [K, N, 2] broadcast over src1 [K, 1, 4] as in src/cuda.rs:1024-1034 (i02 = i12 / (ne12/ne02))."""
-    rng = np.random.default_rng(2)
-    k, n = 256, 48
-    w = oracle.quantize_q4_0((rng.standard_normal((2, n, k)) * 0.02).astype(np.float32))
-    x = rng.standard_normal((4, 1, k)).astype(np.float32)
-    a = g.Tensor.from_raw(w, [k, n, 2], g.Q4_0, gpu)
-    b = g.Tensor.from_raw(x, [k, 1, 4], g.F32, gpu)
-    d = g.Tensor.zeros([n, 1, 4], g.F32, gpu)
+@pytest.mark.parametrize("k,n,ne02,ne12", [(256, 48, 2, 4), (128, 40, 1, 11), (96, 8, 3, 3), (4096, 64, 4, 8)])
+def test_cuda_matmul_batched_broadcast(gpu, k, n, ne02, ne12):
+    """src0 [K, N, ne02] broadcast over src1 [K, 1, ne12] as in src/cuda.rs:1024-1034 (i02 = i12 / (ne12/ne02)):
+    slices in one grouped launch per eight when the shape allows (K % 64 == 0), one launch per slice otherwise."""
+    rng = np.random.default_rng(2 + k)
+    w = oracle.quantize_q4_0((rng.standard_normal((ne02, n, k)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((ne12, 1, k)).astype(np.float32)
+    a = g.Tensor.from_raw(w, [k, n, ne02], g.Q4_0, gpu)
+    b = g.Tensor.from_raw(x, [k, 1, ne12], g.F32, gpu)
+    d = g.Tensor.zeros([n, 1, ne12], g.F32, gpu)
     g.galois_matmul(a, b, d)
-    got = d.to_cpu_tensor().reshape(4, n)
-    for i in range(4):
-        ref = oracle.mul_mat_q4_0_f32(w[i // 2], x[i, 0])
+    got = d.to_cpu_tensor().reshape(ne12, n)
+    for i in range(ne12):
+        ref = oracle.mul_mat_q4_0_f32(w[i // (ne12 // ne02)], x[i, 0])
         emax, _ = npref.rel_err(got[i], ref)
-        assert emax < 1e-4
+        assert emax < 1e-4, i
 
 
 def test_cuda_rmsnorm_rope_softmax(gpu):
