@@ -39,7 +39,7 @@ ROTATE_BYTES = 1200 << 20
 # HBM bytes per grouped launch (the four products) measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE on
 # this workload, each scaled by what the same counter reads for a device-to-device copy of known size
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); see profiles/gemv_q4_0_group__llama7b_gemv_set.md
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 134971699
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 135045120
 
 
 def q4_bytes(k, n):
@@ -352,7 +352,9 @@ def main():
         for i in range(20):
             f(i)
         us = timed(dev, f, 200, reps=5) / 200 * 1e3
-        per_shape.append({"K": k, "N": n, "us": round(us, 3), "weight_GBps": round(q4_bytes(k, n) / us / 1e3, 1),
+        us_graph = timed_graph(dev, f, 200) / 200 * 1e3   # the same launches replayed from a HIP graph: no host in the loop
+        per_shape.append({"K": k, "N": n, "us": round(us, 3), "us_graph_replay": round(us_graph, 3),
+                          "weight_GBps": round(q4_bytes(k, n) / us / 1e3, 1),
                           "hbm_frac": round(q4_bytes(k, n) / us / 1e3 / HBM_PEAK_GBPS, 4)})
 
     extra = {"device": info,
