@@ -233,7 +233,8 @@ def decode_step_bench(dev, reps, with_graph=True):
                 "l2_rel": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
 
     for name, fused in (("eager_one_kernel_per_op", 0), ("eager_fused_norm_and_silu", 1), ("eager_grouped_gemv", 2),
-                        ("eager_grouped_gemv_fused_attention", 3), ("eager_split_norms", 4)):
+                        ("eager_grouped_gemv_fused_attention", 3), ("eager_split_norms", 4),
+                        ("eager_qkv_and_attention_in_one_launch", 5)):
         dec.time_steps(tok, n_past, fused, 3)
         ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
         res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
@@ -241,13 +242,15 @@ def decode_step_bench(dev, reps, with_graph=True):
     if not with_graph:
         dec.close()
         return res
-    dec.capture(tok, n_past, 4)
-    dec.time_replays(3)
-    ms = min(dec.time_replays(reps) for _ in range(3)) / reps
-    res["hip_graph_split_norms"] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4),
-                              "tokens_per_s": round(1e3 / ms, 1),
-                              "GBps": round((weight_bytes + kv_bytes) / ms / 1e6, 1),
-                              "hbm_frac": round((weight_bytes + kv_bytes) / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    graph_logits = {}
+    for name, fused in (("hip_graph_split_norms", 4), ("hip_graph_qkv_and_attention_in_one_launch", 5)):
+        dec.capture(tok, n_past, fused)
+        dec.time_replays(3)
+        ms = min(dec.time_replays(reps) for _ in range(3)) / reps
+        res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
+                     "GBps": round((weight_bytes + kv_bytes) / ms / 1e6, 1),
+                     "hbm_frac": round((weight_bytes + kv_bytes) / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        graph_logits[name] = dec.logits().astype(np.float64)
     logits = dec.logits()
     res["logits_finite"] = bool(np.all(np.isfinite(logits)))
     # the 32-layer logits of the fused plans and of the graph replay against the one-kernel-per-op plan (every op its
@@ -255,20 +258,22 @@ def decode_step_bench(dev, reps, with_graph=True):
     res["logits_vs_one_kernel_per_op"] = {
         "grouped_gemv_fused_attention": cross(plan_logits[3], plan_logits[0]),
         "split_norms": cross(plan_logits[4], plan_logits[0]),
-        "hip_graph_split_norms": cross(logits.astype(np.float64), plan_logits[0])}
+        "qkv_and_attention_in_one_launch": cross(plan_logits[5], plan_logits[0]),
+        **{k: cross(v, plan_logits[0]) for k, v in graph_logits.items()}}
     res["logits_within_1e-4"] = bool(all(v["max_rel"] < 1e-4 and v["l2_rel"] < 1e-4
                                          for v in res["logits_vs_one_kernel_per_op"].values()))
     dec.close()
     # the same step with the KV cache in f16 (the form the reference keeps it in on the GPU): half the cache bytes
     dec, _ = make_decoder(True)
-    dec.time_steps(tok, n_past, 4, 3)
-    ms = min(dec.time_steps(tok, n_past, 4, reps) for _ in range(3)) / reps
     b16 = weight_bytes + kv_bytes // 2
-    res["eager_split_norms_f16_kv"] = {
-        "launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
-        "algorithmic_bytes_per_token": b16, "GBps": round(b16 / ms / 1e6, 1),
-        "hbm_frac": round(b16 / ms / 1e6 / HBM_PEAK_GBPS, 4),
-        "logits_finite": bool(np.all(np.isfinite(dec.logits())))}
+    for name, fused in (("eager_split_norms_f16_kv", 4), ("eager_qkv_and_attention_in_one_launch_f16_kv", 5)):
+        dec.time_steps(tok, n_past, fused, 3)
+        ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
+        res[name] = {
+            "launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
+            "algorithmic_bytes_per_token": b16, "GBps": round(b16 / ms / 1e6, 1),
+            "hbm_frac": round(b16 / ms / 1e6 / HBM_PEAK_GBPS, 4),
+            "logits_finite": bool(np.all(np.isfinite(dec.logits())))}
     dec.close()
     return res
 

@@ -244,6 +244,14 @@ class Device:
                                                                 _ptr(v_cache), _ptr(out), n_head, head_dim, n_past,
                                                                 _ptr(pos), freq_scale, theta_scale, scale))
 
+    def qkv_attn_decode(self, items, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale, scale,
+                        kv_f16=False):
+        """The three q | k | v products (gemv_items of length 3) and the decode attention in one launch."""
+        arr = items if isinstance(items, C.Array) else self.gemv_items(items)
+        fn = self._lib.galois_hip_qkv_attn_decode_f16kv if kv_f16 else self._lib.galois_hip_qkv_attn_decode_f32
+        self._check(fn(self._ctx, arr, _ptr(k_cache), _ptr(v_cache), _ptr(out), n_head, head_dim, n_past, _ptr(pos),
+                       freq_scale, theta_scale, scale))
+
     def attn_decode_f16kv(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
                           scale):
         self._check(self._lib.galois_hip_attn_decode_f16kv(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),

@@ -17,7 +17,8 @@ struct galois_hip_ctx {
     size_t ws_bytes;
     std::vector<void *> ws_retired;  // outgrown workspaces: a graph captured earlier may still point into them
     void *scratch;    // fixed block made at creation: partial sums of the split f32 matmul, partial results of the decode attention
-    unsigned *attn_done;  // GH_ATTN_HEADS counters of the decode attention (splits finished per head), zero between calls
+    unsigned *attn_done;  // 4 x GH_ATTN_HEADS counters, zero between calls: splits finished per head (decode attention), then
+                          // per head the workgroups that have stored its q, its k, its v (the launch that carries both)
     void *attn_static;    // this device's copy of the decode attention's static scratch (attn_decode.hip), found at creation
     bool capturing;   // between graph_begin_capture and graph_end_capture: nothing may allocate or block
     char last_error[256];

@@ -49,8 +49,8 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     const size_t scratch_bytes = GH_PARTIAL_FLOATS * sizeof(float);
     e = hipMalloc(&ctx->scratch, scratch_bytes);
     if (e == hipSuccess) e = hipMemsetAsync(ctx->scratch, 0, scratch_bytes, ctx->stream);
-    if (e == hipSuccess) e = hipMalloc((void **)&ctx->attn_done, GH_ATTN_HEADS * sizeof(unsigned));
-    if (e == hipSuccess) e = hipMemsetAsync(ctx->attn_done, 0, GH_ATTN_HEADS * sizeof(unsigned), ctx->stream);
+    if (e == hipSuccess) e = hipMalloc((void **)&ctx->attn_done, 4 * GH_ATTN_HEADS * sizeof(unsigned));
+    if (e == hipSuccess) e = hipMemsetAsync(ctx->attn_done, 0, 4 * GH_ATTN_HEADS * sizeof(unsigned), ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess && gh_attn_static_init(ctx) != GALOIS_HIP_OK) e = hipErrorNotFound;
     if (e != hipSuccess) {

@@ -16,6 +16,7 @@
 // and the f16 weight scale d.
 #include "common.h"
 #include "gemv_xprep.h"
+#include "attn_decode_body.h"
 
 namespace {
 
@@ -404,9 +405,10 @@ struct gg_args {
 // barrier before the preparation.
 // OUT2: the launch also writes result * scale2 and the workgroup's sum of squares of the result.
 // MAXI: products the selects look at (4 keeps all of their operands in scalar registers at once).
-template <int L, int R, int WAVES, int PG, int OCC, int NORM_MODE, int MAXI, bool OUT2>
-__global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args a) {
-    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+// COHERENT: the results go out as device-coherent stores, for readers in the same launch on other XCDs.
+// item / item_block: which product the workgroup served and its index among that product's workgroups.
+template <int L, int R, int WAVES, int PG, int NORM_MODE, int MAXI, bool OUT2, bool COHERENT>
+__device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, int &item, int &item_block) {
     __shared__ float red[WAVES];
     __shared__ float red2[WAVES];
     constexpr int SD = slot_lds<L>::dwords;
@@ -458,6 +460,7 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
     typedef const __attribute__((address_space(1))) float *global_floats;
     const uint8_t *const W = (const uint8_t *)(global_bytes)W_bits, *const W2 = (const uint8_t *)(global_bytes)W2_bits;
     const float *const xg = (const float *)(global_floats)x_bits;
+    item = ii, item_block = (int)blockIdx.x - first_blk;
     const bool dual = W2 != nullptr;
     const int rw = dual ? R / 2 : R;  // rows per wave and group
     // the workgroup's waves cover WAVES * rw consecutive rows: neighbouring waves read neighbouring rows
@@ -675,7 +678,10 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             typedef __attribute__((address_space(1))) float *global_out;
             const float *res = (const float *)(global_floats)res_bits;
             if (res) out += res[row0 + lane];
-            ((float *)(global_out)dst_bits)[row0 + lane] = out;
+            if (COHERENT)
+                __hip_atomic_store((float *)(global_out)dst_bits + row0 + lane, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else
+                ((float *)(global_out)dst_bits)[row0 + lane] = out;
             if (OUT2) {
                 if (dst2_bits)
                     ((float *)(global_out)dst2_bits)[row0 + lane] = out * scale2_first;
@@ -695,6 +701,13 @@ __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args
             ((float *)(global_out)ssq_bits)[(int)blockIdx.x - first_blk] = tot;
         }
     }
+}
+
+template <int L, int R, int WAVES, int PG, int OCC, int NORM_MODE, int MAXI, bool OUT2>
+__global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args a) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    int item, item_block;
+    gemv_group_wg<L, R, WAVES, PG, NORM_MODE, MAXI, OUT2, false>(a, lds, item, item_block);
 }
 
 template <int L, int R, int G, int WAVES, int OCC>
@@ -761,14 +774,25 @@ void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, int n_items, unsign
         launch_group_cfg<L, R, WAVES, OCC, GG_MAX>(ctx, a, blocks, max_slots, mode, out2);
 }
 
-int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what) {
+// What a group launch needs besides the kernel arguments.
+struct gg_plan {
+    int32_t max_slots = 0;
+    int mode = 0;       // 0 plain, 1 normalising, 2 pre-weighted activations + partial sums of squares
+    bool out2 = false;
+    bool small = false;  // few rows per CU: 16 waves x 1 slot
+    int64_t blocks = 0;
+};
+
+// Checks the items and fills the kernel arguments and the plan.  wide_only: the caller runs the 8-wave x 2-slot
+// shape whatever the row count (a launch that also carries other work).
+int32_t prepare_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what, gg_args &a,
+                      gg_plan &plan, bool wide_only) {
     GH_REQUIRE(ctx, items != nullptr, GALOIS_HIP_E_NULL, what);
     GH_REQUIRE(ctx, n_items >= 1 && n_items <= GG_MAX, GALOIS_HIP_E_SHAPE, "gemv group: 1 to 8 products per call");
-    gg_args a;
     memset(&a, 0, sizeof(a));
     int32_t max_slots = 0;
     int64_t rows = 0;
-    int mode = 0;      // 0 plain, 1 normalising, 2 pre-weighted activations + partial sums of squares
+    int mode = 0;
     bool out2 = false;
     for (int i = 0; i < GG_MAX; i++) a.blk0[i] = 0x7FFFFFFF;
     for (int i = 0; i < n_items; i++) {
@@ -809,7 +833,7 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
     // LLaMA-7B shape.
     bool any_dual = false;
     for (int i = 0; i < n_items; i++) any_dual |= items[i].vx_up != nullptr;
-    const bool small = !any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16;
+    const bool small = !wide_only && !any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16;
     const int slots_per_wg = 16;  // WAVES * R of both shapes
     int64_t blocks = 0;
     for (int i = 0; i < n_items; i++) {
@@ -818,11 +842,121 @@ int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int
         blocks += (items[i].nrows + rows_per_wg - 1) / rows_per_wg;
         GH_REQUIRE(ctx, blocks < 0x7FFFFFFF, GALOIS_HIP_E_SHAPE, "gemv group: too many rows");
     }
+    plan.max_slots = max_slots, plan.mode = mode, plan.out2 = out2, plan.small = small, plan.blocks = blocks;
+    return GALOIS_HIP_OK;
+}
+
+int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what) {
+    gg_args a;
+    gg_plan plan;
+    const int32_t st = prepare_group(ctx, items, n_items, what, a, plan, false);
+    if (st != GALOIS_HIP_OK) return st;
     GH_BIND(ctx);
-    if (small)
-        launch_group_cfg<5, 1, 16, 4>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
+    if (plan.small)
+        launch_group_cfg<5, 1, 16, 4>(ctx, a, n_items, (unsigned)plan.blocks, plan.max_slots, plan.mode, plan.out2);
     else
-        launch_group_cfg<5, 2, 8, 6>(ctx, a, n_items, (unsigned)blocks, max_slots, mode, out2);
+        launch_group_cfg<5, 2, 8, 6>(ctx, a, n_items, (unsigned)plan.blocks, plan.max_slots, plan.mode, plan.out2);
+    GH_LAUNCH_CHECK(ctx, what);
+}
+
+// ---------------------------------------------------------------------------------------
+// The q | k | v products and the decode attention in one launch.
+//
+// Issued as two launches the attention starts when the last product row is out, pays a launch gap, and then spends
+// its first microseconds requesting the cache; its own end is a chain of dependent round trips (split records,
+// counter, merge) during which the memory system idles.  Here the grid is the products' workgroups followed by the
+// attention's: workgroups are handed out in index order, so the attention workgroups take the slots the products
+// free, request their cache rows while the last products still stream, and wait (bounded) only for the 128 floats
+// of their head's q -- the workgroups of the last split, which holds position n_past, also for k and v; whatever a
+// workgroup waits for belongs to workgroups ahead of it in the grid, which are running or done.  A product workgroup
+// stores its 16 rows with device-coherent stores, waits for them, and counts itself on the counter of the head they
+// belong to.  (Measured: with the attention workgroups of the earlier splits placed right behind the q product, so
+// that they are resident from the start, the launch takes twice as long -- the k and v products and then the last
+// split queue up behind them, and the last split's whole latency lands at the end.)
+template <typename CT>
+struct fa_args {
+    CT *kc, *vc;
+    float *part, *out;
+    unsigned *done, *ready;
+    const int32_t *pos;
+    int32_t H, L, S, gemv_blocks;
+    uint32_t target;
+    float freq_scale, theta_scale, scale;
+};
+constexpr int FA_WAVES = 8, FA_HEAD_DIM = 128;
+
+template <int PG, int NORM_MODE, typename CT>
+__global__ __launch_bounds__(FA_WAVES * 64, 4) void qkv_attn_decode_fused(const gg_args a, const fa_args<CT> b) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    if ((int)blockIdx.x < b.gemv_blocks) {
+        int item, item_block;
+        gemv_group_wg<5, 2, FA_WAVES, PG, NORM_MODE, 4, false, true>(a, lds, item, item_block);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows are out
+        __syncthreads();
+        if (threadIdx.x == 0) atomicAdd(b.ready + item * b.H + item_block / (FA_HEAD_DIM / (FA_WAVES * 2)), 1u);
+    } else {
+        // split-major order: the last split, whose workgroups wait for all three products, comes last
+        const int t = (int)blockIdx.x - b.gemv_blocks;
+        attn_decode_wg<FA_HEAD_DIM / 4, CT, FA_WAVES * 64, true>(a.dst[0], a.dst[1], a.dst[2], b.kc, b.vc, b.part, b.done, b.out,
+                                                                 b.H, b.L, b.pos, b.freq_scale, b.theta_scale, b.scale,
+                                                                 t % b.H, t / b.H, b.S, b.ready, b.target);
+    }
+}
+
+template <typename CT>
+int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, CT *k_cache, CT *v_cache, float *out,
+                        int32_t n_head, int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
+                        float theta_scale, float scale, const char *what) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, items && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, head_dim == FA_HEAD_DIM, GALOIS_HIP_E_UNSUPPORTED, "qkv_attn_decode: head_dim 128");
+    GH_REQUIRE(ctx, n_head > 0 && n_head <= GH_ATTN_HEADS && n_past >= 0 && n_past < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
+               "qkv_attn_decode: n_head in 1..65536, n_past >= 0");
+    GH_REQUIRE(ctx, gh_aligned(k_cache, 16) && gh_aligned(v_cache, 16) && gh_aligned(out, 16) && gh_aligned(pos, 4),
+               GALOIS_HIP_E_ALIGN, "qkv_attn_decode: 16-byte aligned caches and output");
+    for (int i = 0; i < 3; i++) {
+        const galois_hip_gemv_item &s = items[i];
+        GH_REQUIRE(ctx, s.nrows == n_head * head_dim && s.ncols == items[0].ncols, GALOIS_HIP_E_SHAPE,
+                   "qkv_attn_decode: three products of n_head * head_dim rows on vectors of one length");
+        GH_REQUIRE(ctx, !s.vx_up && !s.residual && !s.dst_scaled && !s.sumsq_out, GALOIS_HIP_E_UNSUPPORTED,
+                   "qkv_attn_decode: plain or normalising products (no pair, residual or second output)");
+        GH_REQUIRE(ctx, gh_aligned(s.dst, 16), GALOIS_HIP_E_ALIGN, "qkv_attn_decode: 16-byte aligned q, k, v");
+    }
+    gg_args a;
+    gg_plan plan;
+    const int32_t st = prepare_group(ctx, items, 3, what, a, plan, true);
+    if (st != GALOIS_HIP_OK) return st;
+    const int L = n_past + 1;
+    const int S = (L + AT_KEYS - 1) / AT_KEYS;
+    GH_REQUIRE(ctx, S <= AT_MAX_SPLITS && (S == 1 || ((int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS)) &&
+                        ctx->scratch != nullptr && ctx->attn_done != nullptr,
+               GALOIS_HIP_E_UNSUPPORTED, "qkv_attn_decode: n_head * ceil((n_past + 1) / 128) * (head_dim + 4) floats of partial "
+                                         "results must fit the context's 4 MB scratch block");
+    GH_REQUIRE(ctx, plan.blocks + (int64_t)n_head * S < 0x7FFFFFFF, GALOIS_HIP_E_SHAPE, "qkv_attn_decode: too many workgroups");
+    fa_args<CT> b;
+    b.kc = k_cache, b.vc = v_cache, b.part = (float *)ctx->scratch, b.out = out;
+    b.done = ctx->attn_done, b.ready = ctx->attn_done + GH_ATTN_HEADS, b.pos = pos;
+    b.H = n_head, b.L = L, b.S = S, b.gemv_blocks = (int32_t)plan.blocks;
+    b.target = FA_HEAD_DIM / (FA_WAVES * 2);  // workgroups of 16 rows per head
+    b.freq_scale = freq_scale, b.theta_scale = theta_scale, b.scale = scale;
+    GH_BIND(ctx);
+    const dim3 grid((unsigned)(plan.blocks + (int64_t)n_head * S)), block(FA_WAVES * 64);
+    size_t lds = (size_t)plan.max_slots * slot_lds<5>::bytes_per_slot;
+    constexpr int PGMAX = (kChunkSlots * 8 + FA_WAVES * 64 - 1) / (FA_WAVES * 64);
+    const bool short_vec = plan.max_slots <= 64;
+    if (plan.mode == 1 && short_vec) lds += (size_t)plan.max_slots * 64 * sizeof(float);  // staged, weighted activations
+#define FA_LAUNCH(PG_, MODE_) \
+    hipLaunchKernelGGL((qkv_attn_decode_fused<PG_, MODE_, CT>), grid, block, lds, ctx->stream, a, b)
+    if (short_vec) {
+        if (plan.mode == 0) FA_LAUNCH(1, 0);
+        else if (plan.mode == 1) FA_LAUNCH(1, 1);
+        else FA_LAUNCH(1, 2);
+    } else {
+        if (plan.mode == 0) FA_LAUNCH(PGMAX, 0);
+        else if (plan.mode == 1) FA_LAUNCH(PGMAX, 1);
+        else FA_LAUNCH(PGMAX, 2);
+    }
+#undef FA_LAUNCH
     GH_LAUNCH_CHECK(ctx, what);
 }
 
@@ -859,4 +993,20 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *
                                                                 int32_t n_items) {
     GH_REQUIRE_CTX(ctx);
     return launch_group(ctx, items, n_items, "dequantize_mul_mat_vec_q4_0_group");
+}
+
+extern "C" int32_t galois_hip_qkv_attn_decode_f32(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, float *k_cache,
+                                                  float *v_cache, float *out, int32_t n_head, int32_t head_dim,
+                                                  int32_t n_past, const int32_t *pos, float freq_scale, float theta_scale,
+                                                  float scale) {
+    return launch_qkv_attn<float>(ctx, qkv, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
+                                  scale, "qkv_attn_decode_f32");
+}
+
+extern "C" int32_t galois_hip_qkv_attn_decode_f16kv(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, void *k_cache,
+                                                    void *v_cache, float *out, int32_t n_head, int32_t head_dim,
+                                                    int32_t n_past, const int32_t *pos, float freq_scale,
+                                                    float theta_scale, float scale) {
+    return launch_qkv_attn<_Float16>(ctx, qkv, (_Float16 *)k_cache, (_Float16 *)v_cache, out, n_head, head_dim, n_past, pos,
+                                     freq_scale, theta_scale, scale, "qkv_attn_decode_f16kv");
 }

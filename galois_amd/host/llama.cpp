@@ -43,11 +43,10 @@ GResult galois_silu_mul(const Tensor &gate, const Tensor &up, Tensor &dst) {
                                               (float *)dst.data(), (int64_t)gate.dim().elem_count()));
 }
 
-GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
+// Checks the products and writes them as the C ABI's items (at most 8); dev receives their device.
+static GResult matvec_items(const std::vector<MatvecItem> &items, galois_hip_gemv_item *it, std::shared_ptr<CudaDevice> &dev) {
     if (items.empty() || items.size() > 8) return err(GError::ShapeError, "galois_matvec_group: 1 to 8 products");
-    galois_hip_gemv_item it[8];
-    memset(it, 0, sizeof(it));
-    std::shared_ptr<CudaDevice> dev;
+    memset(it, 0, 8 * sizeof(*it));
     for (size_t i = 0; i < items.size(); i++) {
         const MatvecItem &m = items[i];
         if (!m.w || !m.x || !m.dst) return err(GError::Unexpected, "galois_matvec_group: w, x and dst are required");
@@ -81,12 +80,20 @@ GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
         it[i].residual = m.residual ? (const float *)m.residual->data() : nullptr;
         it[i].dst = (float *)m.dst->data(), it[i].ncols = (int32_t)K, it[i].nrows = (int32_t)N, it[i].norm_eps = m.eps;
     }
+    return GError{};
+}
+
+GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
+    galois_hip_gemv_item it[8];
+    std::shared_ptr<CudaDevice> dev;
+    G_TRY(matvec_items(items, it, dev));
     return dev->check(galois_hip_dequantize_mul_mat_vec_q4_0_group(dev->ctx(), it, (int32_t)items.size()));
 }
 
-GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
-                           Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale) {
-    std::shared_ptr<CudaDevice> dev;
+// The checks both attention calls share; dev receives the tensors' device.
+static GResult attn_check(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
+                          Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past,
+                          std::shared_ptr<CudaDevice> &dev) {
     for (const Tensor *t : {&q, &k, &v, (const Tensor *)&k_cache, (const Tensor *)&v_cache, &pos, (const Tensor *)&out}) {
         if (!t->device().is_gpu()) return err(GError::Unimplemented, "galois_attn_decode: Gpu tensors only");
         if (!dev) dev = t->device().gpu;
@@ -103,6 +110,14 @@ GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Te
         out.dim().elem_count() != E || k_cache.dim().shape[0] != E || v_cache.dim().shape[0] != E || pos.dim().elem_count() != 1 ||
         n_past < 0 || (size_t)n_past >= k_cache.dim().shape[1] || (size_t)n_past >= v_cache.dim().shape[1])
         return err(GError::ShapeError, "galois_attn_decode: q, k, v, out of n_head * n_dims elements, caches [that, n_ctx], n_past < n_ctx");
+    return GError{};
+}
+
+GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
+                           Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale) {
+    std::shared_ptr<CudaDevice> dev;
+    G_TRY(attn_check(op, q, k, v, k_cache, v_cache, pos, out, n_head, n_past, dev));
+    const size_t E = q.dim().elem_count();
     const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);  // as galois_rope_custom derives it (src/cuda.rs:1327)
     if (k_cache.dtype() == GGmlType::F16)
         return dev->check(galois_hip_attn_decode_f16kv(dev->ctx(), (const float *)q.data(), (const float *)k.data(),
@@ -112,6 +127,25 @@ GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Te
     return dev->check(galois_hip_attn_decode_f32(dev->ctx(), (const float *)q.data(), (const float *)k.data(), (const float *)v.data(),
                                                  (float *)k_cache.data(), (float *)v_cache.data(), (float *)out.data(), (int32_t)n_head,
                                                  (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
+}
+
+GResult galois_qkv_attn_decode(const RopeCustomOption &op, const std::vector<MatvecItem> &qkv, Tensor &k_cache, Tensor &v_cache,
+                               const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale) {
+    if (qkv.size() != 3) return err(GError::ShapeError, "galois_qkv_attn_decode: the three products q, k, v");
+    galois_hip_gemv_item it[8];
+    std::shared_ptr<CudaDevice> dev, adev;
+    G_TRY(matvec_items(qkv, it, dev));
+    G_TRY(attn_check(op, *qkv[0].dst, *qkv[1].dst, *qkv[2].dst, k_cache, v_cache, pos, out, n_head, n_past, adev));
+    if (adev != dev) return err(GError::Unimplemented, "galois_qkv_attn_decode: one device");
+    const size_t E = out.dim().elem_count();
+    const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);
+    if (k_cache.dtype() == GGmlType::F16)
+        return dev->check(galois_hip_qkv_attn_decode_f16kv(dev->ctx(), it, k_cache.data(), v_cache.data(), (float *)out.data(),
+                                                           (int32_t)n_head, (int32_t)(E / n_head), n_past,
+                                                           (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
+    return dev->check(galois_hip_qkv_attn_decode_f32(dev->ctx(), it, (float *)k_cache.data(), (float *)v_cache.data(),
+                                                     (float *)out.data(), (int32_t)n_head, (int32_t)(E / n_head), n_past,
+                                                     (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
 }
 
 static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t ne1 = 0, size_t ne2 = 0) {
@@ -204,6 +238,8 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
         return err(GError::Unimplemented, "LlamaDecoder: the grouped launch plans (fused >= 2) need n_embd and n_ff to be "
                                           "multiples of 64 no larger than 12288; use fused = 0 or 1");
     const size_t E = hp_.n_embd, H = hp_.n_head, D = E / H, L = (size_t)n_past + 1, C = hp_.n_ctx;
+    if (fused >= 5 && D != 128)
+        return err(GError::Unimplemented, "LlamaDecoder: the launch that carries q | k | v and the attention (fused = 5) needs heads of 128");
     RopeCustomOption rope;
     rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;
     size_t ops = 0;
@@ -235,6 +271,7 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
     for (Layer &l : layers_) {
         const size_t li = (size_t)(&l - &layers_[0]);
         const bool split = fused >= 4;       // norms split over producer and consumer launches
+        const bool qkv_attn = fused >= 5;    // the three projections and the attention in one launch
         if (grouped) {  // rms_norm * weight + the three projections: one launch
             MatvecItem mq = item(l.wq, x_, q_), mk_ = item(l.wk, x_, k_), mv = item(l.wv, x_, v_);
             if (split && li > 0) {  // the previous layer's last launch left x * attn_norm in a_ and the sums of squares of x
@@ -243,7 +280,12 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
             } else {
                 mq.norm_weight = mk_.norm_weight = mv.norm_weight = &l.attn_norm;
             }
-            G_TRY(galois_matvec_group({mq, mk_, mv})); ops++;
+            if (qkv_attn) {
+                G_TRY(galois_qkv_attn_decode(rope, {mq, mk_, mv}, l.k_cache, l.v_cache, pos_, ao_, H, n_past, *(const float *)scale_.data()));
+            } else {
+                G_TRY(galois_matvec_group({mq, mk_, mv}));
+            }
+            ops++;
         } else {
             G_TRY(norm(x_, l.attn_norm, a_));
             G_TRY(galois_matmul(l.wq, a_, q_));
@@ -251,8 +293,10 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
             G_TRY(galois_matmul(l.wv, a_, v_)); ops += 3;
         }
         if (fused >= 3) {  // the eight attention ops as one launch, then the grouped tail of the layer
-            G_TRY(galois_attn_decode(rope, q_, k_, v_, l.k_cache, l.v_cache, pos_, ao_, H, n_past, *(const float *)scale_.data()));
-            ops++;
+            if (!qkv_attn) {
+                G_TRY(galois_attn_decode(rope, q_, k_, v_, l.k_cache, l.v_cache, pos_, ao_, H, n_past, *(const float *)scale_.data()));
+                ops++;
+            }
             MatvecItem mo = item(l.wo, ao_, x1_);
             mo.residual = &x_;
             if (split) mo.dst_scaled = &f_, mo.scale_weight = &l.ffn_norm, mo.sumsq_out = &ssq1_;

@@ -41,6 +41,8 @@ class LlamaDecoder {
     // fused = 4 splits the norms that follow a residual add over the launch that produces the residual stream (it
     // also writes the stream times the next norm weight and its partial sums of squares) and the launch that consumes
     // it (it fetches one vector instead of two and waits for no reduction): the same 5 launches per layer.
+    // fused = 5 sends the q | k | v products and the attention out as one launch (galois_qkv_attn_decode; heads of
+    // 128): 4 launches per layer.
     // fused >= 3 are the plans that run with an f16 KV cache.
     GResult decode(int32_t token, int32_t n_past, int fused);
     // Records the same step as a graph / replays the recorded step.
@@ -94,5 +96,10 @@ GResult galois_matvec_group(const std::vector<MatvecItem> &items);
 // by `scale`, soft_max over the n_past + 1 keys and out = V p, for n_head heads of q.dim / n_head elements.
 GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                            Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale);
+
+// The three products q | k | v (as galois_matvec_group takes them; plain or normalising) and the attention that
+// consumes them (galois_attn_decode on their dst tensors) in one launch (galois_hip_qkv_attn_decode_f32 / _f16kv).
+GResult galois_qkv_attn_decode(const RopeCustomOption &op, const std::vector<MatvecItem> &qkv, Tensor &k_cache, Tensor &v_cache,
+                               const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale);
 
 }  // namespace galois

@@ -270,6 +270,22 @@ int32_t galois_hip_attn_decode_f16kv(galois_hip_ctx *ctx, const float *q, const 
                                      void *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
                                      const int32_t *pos, float freq_scale, float theta_scale, float scale);
 
+/* The q | k | v products of a decode step (three CudaMatMul launches, src/cuda.rs:1011-1034, with whatever
+ * normalisation galois_hip_dequantize_mul_mat_vec_q4_0_group folds in) and the attention that consumes them
+ * (galois_hip_attn_decode_f32 / _f16kv above) as ONE launch: qkv[0..2] are the three products, whose dst are the
+ * q, k and v vectors of n_head * head_dim floats (written as by the group call, and read by the attention part).
+ * The attention's workgroups follow the products' in the grid, request their cache rows while the last products
+ * still stream, and wait -- bounded -- only for their own head's rows of q (k and v where position n_past lives);
+ * should a wait ever run out, that head's output is NaN.  q, k, v and the appended cache rows equal those of the two
+ * calls issued one after the other bit for bit, the output up to the order of its f32 sums.  head_dim 128; the products are plain or normalising (no vx_up, residual, dst_scaled, sumsq_out); dst
+ * 16-byte aligned; limits of both calls apply. */
+int32_t galois_hip_qkv_attn_decode_f32(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, float *k_cache,
+                                       float *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
+                                       const int32_t *pos, float freq_scale, float theta_scale, float scale);
+int32_t galois_hip_qkv_attn_decode_f16kv(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, void *k_cache,
+                                         void *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
+                                         const int32_t *pos, float freq_scale, float theta_scale, float scale);
+
 #ifdef __cplusplus
 }
 #endif

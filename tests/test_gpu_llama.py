@@ -91,12 +91,12 @@ def test_decode_step_matches_oracle_with_a_filled_cache(gdev):
     dec = g.LlamaDecoder(gdev, **hp)
     _load(dec, w, kc, vc)
     ref = _ref_step(w, hp, kc.copy(), vc.copy(), 123, n_past)
-    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1), (3, 5, 1), (4, 5, 1)):
+    for fused, per_layer, tail in ((0, 23, 3), (1, 20, 2), (2, 12, 1), (3, 5, 1), (4, 5, 1), (5, 4, 1)):
         _load(dec, w, kc, vc)
         dec.decode(123, n_past, fused)
         _check(dec.logits(), ref, 1e-4)
         # launches: embedding lookup + per layer + final norm and lm head (fused = 2: grouped products, 12 per layer;
-        # fused = 3: attention in one launch too while n_past + 1 <= 128 keys, two beyond)
+        # fused = 3: attention in one launch too; fused = 5: q | k | v and the attention share a launch)
         assert dec.ops_per_step() == 1 + hp["n_layer"] * per_layer + tail
     # the step wrote row n_past of both caches and nothing else
     kc_ref, vc_ref = kc.copy(), vc.copy()
@@ -119,9 +119,9 @@ def test_decode_from_an_empty_cache_over_several_tokens(gdev):
     _load(dec, w)
     kc = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float32)
     vc = np.zeros_like(kc)
-    for n_past, tok in enumerate([1, 400, 17, 17, 511]):
+    for n_past, tok in enumerate([1, 400, 17, 17, 511, 3, 250]):
         ref = _ref_step(w, hp, kc, vc, tok, n_past)
-        dec.decode(tok, n_past, (0, 3, 2, 4, 1)[n_past])   # every launch plan in turn, on one cache
+        dec.decode(tok, n_past, (0, 3, 2, 4, 1, 5, 5)[n_past])   # every launch plan in turn, on one cache
         _check(dec.logits(), ref, 1e-4)
     dec.close()
 
@@ -136,16 +136,16 @@ def test_decode_with_an_f16_kv_cache(gdev):
     _load(dec, w)
     kc = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float32)
     vc = np.zeros_like(kc)
-    for n_past, tok in enumerate([5, 300, 41, 41]):
+    for n_past, tok in enumerate([5, 300, 41, 41, 77, 8]):
         # the oracle's step appends f32 rows; this step's own attention must already see them rounded
         ref = _ref_step(w, hp, kc, vc, tok, n_past, round_kv=True)
-        dec.decode(tok, n_past, 3)
+        dec.decode(tok, n_past, (3, 3, 4, 3, 5, 5)[n_past])
         _check(dec.logits(), ref, 2e-4)
     kg = dec.tensor("k_cache", 1).to_cpu_tensor()
-    assert kg.dtype == np.float16 and np.array_equal(kg[4:], np.zeros_like(kg[4:])) and np.any(kg[3] != 0)
-    _check(kg[:4].astype(np.float32), kc[1][:4], 1e-3)
+    assert kg.dtype == np.float16 and np.array_equal(kg[6:], np.zeros_like(kg[6:])) and np.any(kg[5] != 0)
+    _check(kg[:6].astype(np.float32), kc[1][:6], 1e-3)
     with pytest.raises(g.GError) as e:
-        dec.decode(1, 4, 2)
+        dec.decode(1, 6, 2)
     assert e.value.kind == "Unimplemented"
     dec.close()
 
@@ -203,21 +203,22 @@ def test_full_width_layers_at_kv_length_2048(gdev):
     vc = rng.standard_normal((2, 2048, 4096)).astype(np.float32)
     dec = g.LlamaDecoder(gdev, **hp)
     ref = _ref_step(w, hp, kc.copy(), vc.copy(), 31999, 2047)
-    for fused in (0, 1, 2, 3, 4):
+    for fused in (0, 1, 2, 3, 4, 5):
         _load(dec, w, kc, vc)
         dec.decode(31999, 2047, fused)
         _check(dec.logits(), ref, 1e-4)
-    _load(dec, w, kc, vc)
-    dec.capture(31999, 2047, 4)
-    for _ in range(2):
-        dec.replay()
-        _check(dec.logits(), ref, 1e-4)
+    for fused in (4, 5):
+        _load(dec, w, kc, vc)
+        dec.capture(31999, 2047, fused)
+        for _ in range(2):
+            dec.replay()
+            _check(dec.logits(), ref, 1e-4)
     dec.close()
     # f16 caches: the oracle's step on the f16 contents, this step's rows rounded before the attention reads them
     kc16, vc16 = kc.astype(np.float16), vc.astype(np.float16)
     dec = g.LlamaDecoder(gdev, kv_f16=True, **hp)
     ref16 = _ref_step(w, hp, kc16.astype(np.float32), vc16.astype(np.float32), 31999, 2047, round_kv=True)
-    for fused in (3, 4):
+    for fused in (3, 4, 5):
         _load(dec, w, kc16, vc16)
         dec.decode(31999, 2047, fused)
         _check(dec.logits(), ref16, 2e-4)

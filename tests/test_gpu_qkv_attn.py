@@ -1,0 +1,76 @@
+"""The launch that carries the q | k | v products and the decode attention together against the same two calls issued
+one after the other: q, k, v and the appended cache rows are bit-equal; the attention's output agrees up to the order
+of its f32 sums (eight waves instead of four share a split's keys): 1e-5 of the largest output, the tolerance of the
+attention's own parity test."""
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dev, H, K, n_past, mode, kv_f16, seed, repeats=1, n_ctx=None):
+    D = 128
+    E = H * D
+    rng = np.random.default_rng(seed)
+    n_ctx = n_ctx or n_past + 1
+    ws = [dev.upload(oracle.quantize_q4_0((rng.standard_normal((E, K)) * 0.05).astype(np.float32))) for _ in range(3)]
+    x = dev.upload(rng.standard_normal(K).astype(np.float32))
+    nw = dev.upload((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    ssq = dev.upload(np.abs(rng.standard_normal((K + 15) // 16)).astype(np.float32) * 16)
+    ct = np.float16 if kv_f16 else np.float32
+    kc0 = rng.standard_normal((n_ctx, E)).astype(ct)
+    vc0 = rng.standard_normal((n_ctx, E)).astype(ct)
+    pos = dev.upload(np.array([n_past], np.int32))
+    fs, ts, scale = 1.0, 10000.0 ** (-2.0 / D), D ** -0.5
+
+    def side():
+        q, k, v = (dev.upload(np.full(E, 3.25, np.float32)) for _ in range(3))
+        items = []
+        for w, d in zip(ws, (q, k, v)):
+            it = {"vx": w, "y": x, "dst": d, "ncols": K, "nrows": E}
+            if mode == 1:
+                it.update(norm_weight=nw, norm_eps=1e-5)
+            elif mode == 2:
+                it.update(sumsq_in=ssq, norm_eps=1e-5)
+            items.append(it)
+        return dict(q=q, k=k, v=v, items=dev.gemv_items(items), kc=dev.upload(kc0), vc=dev.upload(vc0),
+                    out=dev.upload(np.full(E + 16, 7.5, np.float32)))
+
+    a, b = side(), side()
+    for r in range(repeats):
+        print("qkv_attn case H=%d K=%d n_past=%d mode=%d f16=%s rep=%d" % (H, K, n_past, mode, kv_f16, r), flush=True)
+        dev.dequantize_mul_mat_vec_q4_0_group(a["items"])
+        attn = dev.attn_decode_f16kv if kv_f16 else dev.attn_decode_f32
+        attn(a["q"], a["k"], a["v"], a["kc"], a["vc"], a["out"], H, D, n_past, pos, fs, ts, scale)
+        dev.qkv_attn_decode(b["items"], b["kc"], b["vc"], b["out"], H, D, n_past, pos, fs, ts, scale, kv_f16=kv_f16)
+        dev.synchronize()
+        for name, n, t in (("q", E, np.float32), ("k", E, np.float32), ("v", E, np.float32), ("out", E + 16, np.float32),
+                           ("kc", kc0.shape, ct), ("vc", vc0.shape, ct)):
+            ra, rb = dev.download(a[name], t, n), dev.download(b[name], t, n)
+            if name == "out":
+                assert np.all(np.isfinite(rb[:E])) and np.all(rb[E:] == 7.5)
+                assert np.max(np.abs(ra[:E] - rb[:E])) <= 1e-5 * np.max(np.abs(ra[:E])), r
+            else:
+                assert np.array_equal(ra.view(np.uint8), rb.view(np.uint8)), (name, r)
+    for s in (a, b):
+        for key in ("q", "k", "v", "kc", "vc", "out"):
+            dev.free(s[key])
+    for buf in ws + [x, nw, ssq, pos]:
+        dev.free(buf)
+
+
+@pytest.mark.parametrize("H,K,n_past,mode,kv_f16", [
+    (2, 256, 0, 0, False), (2, 256, 5, 1, False), (3, 320, 130, 2, False), (4, 256, 127, 1, True),
+    (2, 5120, 300, 1, False), (2, 4160, 300, 2, True), (2, 4160, 40, 0, False),
+    (32, 4096, 2047, 2, False), (32, 4096, 2047, 1, False), (32, 4096, 2047, 2, True), (32, 4096, 2300, 0, False)])
+def test_qkv_attn_equals_the_two_calls(dev, H, K, n_past, mode, kv_f16):
+    _case(dev, H, K, n_past, mode, kv_f16, seed=H * 1000 + n_past)
+
+
+def test_qkv_attn_repeated_calls(dev):
+    """Counters return to zero: the same launch again and again, and a different head count after it."""
+    _case(dev, 32, 4096, 1500, 2, False, seed=5, repeats=6)
+    _case(dev, 5, 256, 700, 1, False, seed=6, repeats=3)
+    _case(dev, 32, 4096, 100, 1, True, seed=7, repeats=3)
