@@ -213,7 +213,14 @@ void launch_vec_krows(galois_hip_ctx *ctx, const AT *a, const float *b, float *d
 bool gh_mul_mat_f16_mfma(galois_hip_ctx *ctx, const _Float16 *a, const float *b, float *dst, int K, int N, int M,
                          int ne02, int ne12, int64_t a_s1, int64_t a_s2);
 
+// gemm_f32_mfma (mul_mat_f32_mfma.hip): many rows of b on the matrix cores in full f32, a contiguous along K or N.
+template <typename AT>
+bool gh_mul_mat_f32_mfma(galois_hip_ctx *ctx, const AT *a, const float *b, float *dst, int K, int N, int M, int ne02,
+                         int ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2);
+
 namespace {
+
+constexpr int kMfmaMinRows = 16;  // rows of b from which the 128-row tiles of the f32 matrix-core kernel pay
 
 template <typename AT>
 int32_t mul_mat_any(galois_hip_ctx *ctx, const AT *a, const float *b, float *dst, int32_t K, int32_t N, int32_t M,
@@ -232,6 +239,8 @@ int32_t mul_mat_any(galois_hip_ctx *ctx, const AT *a, const float *b, float *dst
     if (F16 && M > 1 && a_s0 == 1 &&
         gh_mul_mat_f16_mfma(ctx, (const _Float16 *)a, b, dst, K, N, M, ne02, ne12, a_s1, a_s2))
         GH_LAUNCH_CHECK(ctx, "mul_mat_f16_f32 launch");
+    if (M >= kMfmaMinRows && gh_mul_mat_f32_mfma<AT>(ctx, a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2))
+        GH_LAUNCH_CHECK(ctx, "mul_mat_f32 launch (matrix cores)");
     const bool vec16 = M == 1 && gh_aligned(a, A16) && gh_aligned(b, 16) && a_s2 % 4 == 0;
     if (a_s0 == 1) {
         const bool fast = vec16 && a_s1 % 4 == 0 && (K == 32 || K == 64 || K == 128 || K == 256);
