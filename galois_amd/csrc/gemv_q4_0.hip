@@ -783,10 +783,11 @@ struct gg_plan {
     int64_t blocks = 0;
 };
 
-// Checks the items and fills the kernel arguments and the plan.  wide_only: the caller runs the 8-wave x 2-slot
-// shape whatever the row count (a launch that also carries other work).
+// Checks the items and fills the kernel arguments and the plan.  wg_slots: 0 = the shape is chosen here (16 slots
+// per workgroup either way); otherwise the caller's kernel has workgroups of that many slots (a launch that also
+// carries other work).
 int32_t prepare_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what, gg_args &a,
-                      gg_plan &plan, bool wide_only) {
+                      gg_plan &plan, int wg_slots) {
     GH_REQUIRE(ctx, items != nullptr, GALOIS_HIP_E_NULL, what);
     GH_REQUIRE(ctx, n_items >= 1 && n_items <= GG_MAX, GALOIS_HIP_E_SHAPE, "gemv group: 1 to 8 products per call");
     memset(&a, 0, sizeof(a));
@@ -833,8 +834,8 @@ int32_t prepare_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, in
     // LLaMA-7B shape.
     bool any_dual = false;
     for (int i = 0; i < n_items; i++) any_dual |= items[i].vx_up != nullptr;
-    const bool small = !wide_only && !any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16;
-    const int slots_per_wg = 16;  // WAVES * R of both shapes
+    const bool small = !wg_slots && !any_dual && (rows + ctx->n_cu - 1) / ctx->n_cu <= 16;
+    const int slots_per_wg = wg_slots ? wg_slots : 16;  // WAVES * R of both shapes
     int64_t blocks = 0;
     for (int i = 0; i < n_items; i++) {
         const int64_t rows_per_wg = items[i].vx_up ? slots_per_wg / 2 : slots_per_wg;
@@ -849,7 +850,7 @@ int32_t prepare_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, in
 int32_t launch_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, int32_t n_items, const char *what) {
     gg_args a;
     gg_plan plan;
-    const int32_t st = prepare_group(ctx, items, n_items, what, a, plan, false);
+    const int32_t st = prepare_group(ctx, items, n_items, what, a, plan, 0);
     if (st != GALOIS_HIP_OK) return st;
     GH_BIND(ctx);
     if (plan.small)
@@ -884,16 +885,18 @@ struct fa_args {
     float freq_scale, theta_scale, scale;
 };
 constexpr int FA_WAVES = 8, FA_HEAD_DIM = 128;
+constexpr int FA_R = 2;  // rows per wave of the products (measured: 4, which makes all products resident at once, 30.7 against 25.3 us)
+static_assert(FA_HEAD_DIM % (FA_WAVES * FA_R) == 0, "a product workgroup's rows belong to one head");
 
 template <int PG, int NORM_MODE, typename CT>
 __global__ __launch_bounds__(FA_WAVES * 64, 4) void qkv_attn_decode_fused(const gg_args a, const fa_args<CT> b) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     if ((int)blockIdx.x < b.gemv_blocks) {
         int item, item_block;
-        gemv_group_wg<5, 2, FA_WAVES, PG, NORM_MODE, 4, false, true>(a, lds, item, item_block);
+        gemv_group_wg<5, FA_R, FA_WAVES, PG, NORM_MODE, 4, false, true>(a, lds, item, item_block);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows are out
         __syncthreads();
-        if (threadIdx.x == 0) atomicAdd(b.ready + item * b.H + item_block / (FA_HEAD_DIM / (FA_WAVES * 2)), 1u);
+        if (threadIdx.x == 0) atomicAdd(b.ready + item * b.H + item_block / (FA_HEAD_DIM / (FA_WAVES * FA_R)), 1u);
     } else {
         // split-major order: the last split, whose workgroups wait for all three products, comes last
         const int t = (int)blockIdx.x - b.gemv_blocks;
@@ -924,7 +927,7 @@ int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, 
     }
     gg_args a;
     gg_plan plan;
-    const int32_t st = prepare_group(ctx, items, 3, what, a, plan, true);
+    const int32_t st = prepare_group(ctx, items, 3, what, a, plan, FA_WAVES * FA_R);
     if (st != GALOIS_HIP_OK) return st;
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
@@ -937,7 +940,7 @@ int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, 
     b.kc = k_cache, b.vc = v_cache, b.part = (float *)ctx->scratch, b.out = out;
     b.done = ctx->attn_done, b.ready = ctx->attn_done + GH_ATTN_HEADS, b.pos = pos;
     b.H = n_head, b.L = L, b.S = S, b.gemv_blocks = (int32_t)plan.blocks;
-    b.target = FA_HEAD_DIM / (FA_WAVES * 2);  // workgroups of 16 rows per head
+    b.target = FA_HEAD_DIM / (FA_WAVES * FA_R);  // product workgroups per head
     b.freq_scale = freq_scale, b.theta_scale = theta_scale, b.scale = scale;
     GH_BIND(ctx);
     const dim3 grid((unsigned)(plan.blocks + (int64_t)n_head * S)), block(FA_WAVES * 64);
