@@ -69,6 +69,27 @@ def test_qkv_attn_equals_the_two_calls(dev, H, K, n_past, mode, kv_f16):
     _case(dev, H, K, n_past, mode, kv_f16, seed=H * 1000 + n_past)
 
 
+def test_qkv_attn_argument_errors(dev):
+    from galois_amd import GaloisHipError
+    rng = np.random.default_rng(1)
+    H, D, K = 2, 128, 256
+    E = H * D
+    w = dev.upload(oracle.quantize_q4_0((rng.standard_normal((E, K)) * 0.05).astype(np.float32)))
+    x, q, kc, out = dev.upload(np.ones(K, np.float32)), dev.alloc(E * 4), dev.alloc(4 * E * 4), dev.alloc(E * 4)
+    pos = dev.upload(np.array([0], np.int32))
+    item = {"vx": w, "y": x, "dst": q, "ncols": K, "nrows": E}
+    ok = [item, item, item]
+    for items, h, d, code in ((ok, H, 64, -5),                                           # heads of 128 only
+                              ([item, item, dict(item, nrows=E - 16)], H, D, -2),        # every product n_head * head_dim rows
+                              ([item, item, dict(item, residual=x)], H, D, -5),          # no residual, pair or second output
+                              (ok, 0, D, -2)):
+        with pytest.raises(GaloisHipError) as ei:
+            dev.qkv_attn_decode(items, kc, kc, out, h, d, 0, pos, 1.0, 0.9, 0.1)
+        assert ei.value.status == code, (ei.value.status, code)
+    for b in (w, x, q, kc, out, pos):
+        dev.free(b)
+
+
 def test_qkv_attn_repeated_calls(dev):
     """Counters return to zero: the same launch again and again, and a different head count after it."""
     _case(dev, 32, 4096, 1500, 2, False, seed=5, repeats=6)
