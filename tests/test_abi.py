@@ -80,7 +80,7 @@ def test_ctypes_argument_lists_match_the_header():
 
 
 def _rust_prototypes():
-    """The extern block of INTEGRATION.md, the binding a maintainer would paste into src/hip.rs."""
+    """The Rust extern block of the integration notes: the binding a maintainer would paste into src/hip.rs."""
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     out = {}
     for name, args, ret in re.findall(r"pub fn (galois_hip_[a-z0-9_]+)\(([^)]*)\)\s*->\s*([^;]+);", text):
