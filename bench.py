@@ -185,8 +185,9 @@ def decode_step_bench(dev, reps, with_graph=True):
     gdev = g.Device.gpu(0)
     seed = [0]
 
-    def make_decoder(kv_f16):
-        dec = g.LlamaDecoder(gdev, kv_f16=kv_f16)   # defaults = the config: 4096 / 32 heads / 11008 / 32000 / 32 layers
+    def make_decoder(kv_f16, head_major=False):
+        seed[0] = 0   # every decoder gets the same weights and the same cache contents
+        dec = g.LlamaDecoder(gdev, kv_f16=kv_f16, kv_head_major=head_major)   # defaults = the config: 4096 / 32 heads / 11008 / 32000 / 32 layers
         hp = dec.hp
         e, f, v, c = hp["n_embd"], hp["n_ff"], hp["n_vocab"], hp["n_ctx"]
         stage = dev.alloc(e * v * 4)
@@ -197,9 +198,11 @@ def decode_step_bench(dev, reps, with_graph=True):
             dev.quantize_row_q4_0(stage, t.data_ptr(), rows * cols)
             dev.synchronize()
 
-        def fill_f32(t, count, mean, scale, f16=False):
+        def fill_f32(t, count, mean, scale, f16=False, cache=False):
             seed[0] += 1
             a = _normal_f32(seed[0], count, scale) + np.float32(mean)
+            if cache and head_major:   # the same elements, kept [n_head][n_ctx][head_dim]
+                a = np.ascontiguousarray(a.reshape(c, hp["n_head"], -1).transpose(1, 0, 2)).ravel()
             t.write(a.astype(np.float16) if f16 else a)
 
         fill_q4(dec.tensor("tok_embd"), v, e)
@@ -213,8 +216,8 @@ def decode_step_bench(dev, reps, with_graph=True):
                 weight_bytes += q4_bytes(cols, rows)
             fill_f32(dec.tensor("attn_norm", i), e, 1.0, 0.1)
             fill_f32(dec.tensor("ffn_norm", i), e, 1.0, 0.1)
-            fill_f32(dec.tensor("k_cache", i), e * c, 0.0, 1.0, kv_f16)
-            fill_f32(dec.tensor("v_cache", i), e * c, 0.0, 1.0, kv_f16)
+            fill_f32(dec.tensor("k_cache", i), e * c, 0.0, 1.0, kv_f16, True)
+            fill_f32(dec.tensor("v_cache", i), e * c, 0.0, 1.0, kv_f16, True)
         dev.free(stage)
         return dec, weight_bytes
 
@@ -262,6 +265,17 @@ def decode_step_bench(dev, reps, with_graph=True):
         **{k: cross(v, plan_logits[0]) for k, v in graph_logits.items()}}
     res["logits_within_1e-4"] = bool(all(v["max_rel"] < 1e-4 and v["l2_rel"] < 1e-4
                                          for v in res["logits_vs_one_kernel_per_op"].values()))
+    dec.close()
+    # the same step with the caches kept [n_head][n_ctx][head_dim]: a head's keys contiguous (same weights, same cache
+    # contents: the logits are compared with the one-kernel-per-op plan of the [n_ctx][n_embd] decoder above)
+    dec, _ = make_decoder(False, True)
+    for name, fused in (("eager_split_norms_head_major_kv", 4), ("eager_qkv_and_attention_in_one_launch_head_major_kv", 5)):
+        dec.time_steps(tok, n_past, fused, 3)
+        ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
+        res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
+                     "GBps": round((weight_bytes + kv_bytes) / ms / 1e6, 1),
+                     "hbm_frac": round((weight_bytes + kv_bytes) / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                     "logits_vs_one_kernel_per_op": cross(dec.logits().astype(np.float64), plan_logits[0])}
     dec.close()
     # the same step with the KV cache in f16 (the form the reference keeps it in on the GPU): half the cache bytes
     dec, _ = make_decoder(True)

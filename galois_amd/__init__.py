@@ -233,30 +233,31 @@ class Device:
                                                        n_table_rows))
 
     def attn_decode_f32(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
-                        scale):
+                        scale, head_major_n_ctx=0):
         self._check(self._lib.galois_hip_attn_decode_f32(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),
                                                          _ptr(v_cache), _ptr(out), n_head, head_dim, n_past, _ptr(pos),
-                                                         freq_scale, theta_scale, scale))
+                                                         freq_scale, theta_scale, scale, head_major_n_ctx))
 
     def attn_decode_f32_static(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale,
-                               theta_scale, scale):
+                               theta_scale, scale, head_major_n_ctx=0):
         self._check(self._lib.galois_hip_attn_decode_f32_static(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),
                                                                 _ptr(v_cache), _ptr(out), n_head, head_dim, n_past,
-                                                                _ptr(pos), freq_scale, theta_scale, scale))
+                                                                _ptr(pos), freq_scale, theta_scale, scale,
+                                                                head_major_n_ctx))
 
     def qkv_attn_decode(self, items, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale, scale,
-                        kv_f16=False):
+                        kv_f16=False, head_major_n_ctx=0):
         """The three q | k | v products (gemv_items of length 3) and the decode attention in one launch."""
         arr = items if isinstance(items, C.Array) else self.gemv_items(items)
         fn = self._lib.galois_hip_qkv_attn_decode_f16kv if kv_f16 else self._lib.galois_hip_qkv_attn_decode_f32
         self._check(fn(self._ctx, arr, _ptr(k_cache), _ptr(v_cache), _ptr(out), n_head, head_dim, n_past, _ptr(pos),
-                       freq_scale, theta_scale, scale))
+                       freq_scale, theta_scale, scale, head_major_n_ctx))
 
     def attn_decode_f16kv(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
-                          scale):
+                          scale, head_major_n_ctx=0):
         self._check(self._lib.galois_hip_attn_decode_f16kv(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),
                                                            _ptr(v_cache), _ptr(out), n_head, head_dim, n_past,
-                                                           _ptr(pos), freq_scale, theta_scale, scale))
+                                                           _ptr(pos), freq_scale, theta_scale, scale, head_major_n_ctx))
 
     def mul_mat_f16_f32(self, a, b, dst, K, N, M, ne02, ne12, a_s0, a_s1, a_s2):
         self._check(self._lib.galois_hip_mul_mat_f16_f32(self._ctx, _ptr(a), _ptr(b), _ptr(dst), K, N, M, ne02, ne12,

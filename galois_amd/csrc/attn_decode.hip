@@ -28,9 +28,11 @@ __global__ __launch_bounds__(AT_THREADS) void attn_decode_partial(const float *_
                                                                   CT *__restrict__ vc, float *__restrict__ part,
                                                                   unsigned *__restrict__ done, float *__restrict__ out, int H, int L,
                                                                   const int32_t *__restrict__ pos, float freq_scale,
-                                                                  float theta_scale, float scale) {
+                                                                  float theta_scale, float scale, int64_t key_stride,
+                                                                  int64_t head_stride) {
     attn_decode_wg<LPR, CT, AT_THREADS, false>(q, k, v, kc, vc, part, done, out, H, L, pos, freq_scale, theta_scale, scale,
-                                               (int)blockIdx.y, (int)blockIdx.x, (int)gridDim.x, nullptr, 0u);
+                                               (int)blockIdx.y, (int)blockIdx.x, (int)gridDim.x, nullptr, 0u, key_stride,
+                                               head_stride);
 }
 
 // Scratch of the entry point that allocates nothing: per-head counters, then the split records.  One copy per
@@ -46,7 +48,8 @@ namespace {
 template <typename CT>
 int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, CT *k_cache, CT *v_cache,
                            float *out, int32_t n_head, int32_t head_dim, int32_t n_past, const int32_t *pos,
-                           float freq_scale, float theta_scale, float scale, const char *what, bool static_scratch = false) {
+                           float freq_scale, float theta_scale, float scale, int32_t head_major_n_ctx, const char *what,
+                           bool static_scratch = false) {
     GH_REQUIRE_CTX(ctx);
     GH_REQUIRE(ctx, q && k && v && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, what);
     GH_REQUIRE(ctx, n_head > 0 && n_head <= 65535 && n_past >= 0 && n_past < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
@@ -55,6 +58,10 @@ int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, 
     GH_REQUIRE(ctx, gh_aligned(q, 16) && gh_aligned(k, 16) && gh_aligned(v, 16) && gh_aligned(k_cache, 16) &&
                         gh_aligned(v_cache, 16) && gh_aligned(out, 16) && gh_aligned(pos, 4),
                GALOIS_HIP_E_ALIGN, "attn_decode: 16-byte aligned vectors and caches");
+    GH_REQUIRE(ctx, head_major_n_ctx == 0 || head_major_n_ctx > n_past, GALOIS_HIP_E_SHAPE,
+               "attn_decode: head_major_n_ctx is 0 or the capacity of a [n_head][n_ctx][head_dim] cache, above n_past");
+    const int64_t key_stride = head_major_n_ctx ? head_dim : (int64_t)n_head * head_dim;
+    const int64_t head_stride = head_major_n_ctx ? (int64_t)head_major_n_ctx * head_dim : head_dim;
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
     float *part;
@@ -78,10 +85,10 @@ int32_t attn_decode_launch(galois_hip_ctx *ctx, const float *q, const float *k, 
     const dim3 grid((unsigned)S, (unsigned)n_head), block(AT_THREADS);
     if (head_dim == 128)
         hipLaunchKernelGGL((attn_decode_partial<32, CT>), grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done,
-                           out, n_head, L, pos, freq_scale, theta_scale, scale);
+                           out, n_head, L, pos, freq_scale, theta_scale, scale, key_stride, head_stride);
     else
         hipLaunchKernelGGL((attn_decode_partial<16, CT>), grid, block, 0, ctx->stream, q, k, v, k_cache, v_cache, part, done,
-                           out, n_head, L, pos, freq_scale, theta_scale, scale);
+                           out, n_head, L, pos, freq_scale, theta_scale, scale, key_stride, head_stride);
     GH_LAUNCH_CHECK(ctx, what);
 }
 
@@ -100,23 +107,23 @@ int32_t gh_attn_static_init(galois_hip_ctx *ctx) {
 extern "C" int32_t galois_hip_attn_decode_f32_static(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
                                                      float *k_cache, float *v_cache, float *out, int32_t n_head,
                                                      int32_t head_dim, int32_t n_past, const int32_t *pos,
-                                                     float freq_scale, float theta_scale, float scale) {
+                                                     float freq_scale, float theta_scale, float scale, int32_t head_major_n_ctx) {
     return attn_decode_launch<float>(ctx, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale,
-                                     theta_scale, scale, "attn_decode_f32_static", true);
+                                     theta_scale, scale, head_major_n_ctx, "attn_decode_f32_static", true);
 }
 
 extern "C" int32_t galois_hip_attn_decode_f32(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
                                               float *k_cache, float *v_cache, float *out, int32_t n_head,
                                               int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
-                                              float theta_scale, float scale) {
+                                              float theta_scale, float scale, int32_t head_major_n_ctx) {
     return attn_decode_launch<float>(ctx, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale,
-                                     theta_scale, scale, "attn_decode_f32");
+                                     theta_scale, scale, head_major_n_ctx, "attn_decode_f32");
 }
 
 extern "C" int32_t galois_hip_attn_decode_f16kv(galois_hip_ctx *ctx, const float *q, const float *k, const float *v,
                                                 void *k_cache, void *v_cache, float *out, int32_t n_head,
                                                 int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
-                                                float theta_scale, float scale) {
+                                                float theta_scale, float scale, int32_t head_major_n_ctx) {
     return attn_decode_launch<_Float16>(ctx, q, k, v, (_Float16 *)k_cache, (_Float16 *)v_cache, out, n_head, head_dim,
-                                        n_past, pos, freq_scale, theta_scale, scale, "attn_decode_f16kv");
+                                        n_past, pos, freq_scale, theta_scale, scale, head_major_n_ctx, "attn_decode_f16kv");
 }

@@ -176,6 +176,9 @@ __device__ __forceinline__ float4 at_load4_coherent(const float *p) {
 
 // The work of one workgroup: split s of head h (S splits per head).  Record of one (head, split) in the scratch
 // block: m, sum, 2 unused floats, then head_dim partial outputs.
+// Cache element (position l, head h, d) lies at l * key_stride + h * head_stride + d: (H * D, D) for caches kept
+// [n_ctx][n_head * head_dim], (D, n_ctx * D) for caches kept [n_head][n_ctx][head_dim], where a workgroup's 128 keys
+// are one contiguous 64 KB instead of 128 pieces of 512 bytes.
 // FUSED: q, k and v are written by other workgroups of the same launch (the q | k | v products); ready[h],
 // ready[H + h], ready[2 H + h] count the workgroups that have stored their rows of head h's q, k, v, and reach
 // `target` when the head's rows are complete.  The cache rows are requested first, then the workgroup waits for q
@@ -187,7 +190,7 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
                                                float *__restrict__ part, unsigned *__restrict__ done,
                                                float *__restrict__ out, int H, int L, const int32_t *__restrict__ pos,
                                                float freq_scale, float theta_scale, float scale, int h, int s, int S,
-                                               unsigned *ready, unsigned target) {
+                                               unsigned *ready, unsigned target, int64_t key_stride, int64_t head_stride) {
     constexpr int D = LPR * 4, RPL = 64 / LPR, WAVES = AT_THREADS / 64;
     constexpr int KEYS = AT_KEYS;
     constexpr int KPW = KEYS / WAVES;     // keys per wave
@@ -202,8 +205,9 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane / LPR, kl = lane % LPR;
     const int l0 = s * KEYS, l1 = min(L, l0 + KEYS), nl = l1 - l0;
-    const size_t E = (size_t)H * D;
-    const size_t hoff = (size_t)h * D + kl * 4;
+    const size_t hoff = (size_t)h * D + kl * 4;                    // in q, k, v, out
+    const size_t coff = (size_t)h * (size_t)head_stride + kl * 4;  // in the caches: element (l, h, d) at l * key_stride + h * head_stride + d
+    const size_t E = (size_t)key_stride;
 
     const int lnew = L - 1;  // the position being appended
     const int kbase = l0 + wave * KPW + sub;
@@ -223,9 +227,9 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
     }
     typename at_raw<CT>::type kv[U], vv[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) kv[u] = at_load4(kc + (size_t)min(kbase + u * RPL, l1 - 1) * E + hoff);
+    for (int u = 0; u < U; u++) kv[u] = at_load4(kc + (size_t)min(kbase + u * RPL, l1 - 1) * E + coff);
 #pragma unroll
-    for (int u = 0; u < U; u++) vv[u] = at_load4(vc + (size_t)min(kbase + u * RPL, l1 - 1) * E + hoff);
+    for (int u = 0; u < U; u++) vv[u] = at_load4(vc + (size_t)min(kbase + u * RPL, l1 - 1) * E + coff);
     float4 knew_raw, vnew, qraw;
     if (!FUSED) {
         knew_raw = *reinterpret_cast<const float4 *>(k + hoff);
@@ -271,8 +275,8 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
         if (min(l, l1 - 1) == lnew) {  // the new key; the lanes that own it write both cache rows
             kf = knew;
             if (l == lnew) {
-                at_store4(kc + (size_t)lnew * E + hoff, knew);
-                at_store4(vc + (size_t)lnew * E + hoff, vnew);
+                at_store4(kc + (size_t)lnew * E + coff, knew);
+                at_store4(vc + (size_t)lnew * E + coff, vnew);
             }
         }
         float acc = kf.x * qv.x;

@@ -883,6 +883,7 @@ struct fa_args {
     int32_t H, L, S, gemv_blocks;
     uint32_t target;
     float freq_scale, theta_scale, scale;
+    int64_t key_stride, head_stride;  // of the caches, in elements
 };
 constexpr int FA_WAVES = 8, FA_HEAD_DIM = 128;
 constexpr int FA_R = 2;  // rows per wave of the products (measured: 4, which makes all products resident at once, 30.7 against 25.3 us)
@@ -902,17 +903,20 @@ __global__ __launch_bounds__(FA_WAVES * 64, 4) void qkv_attn_decode_fused(const 
         const int t = (int)blockIdx.x - b.gemv_blocks;
         attn_decode_wg<FA_HEAD_DIM / 4, CT, FA_WAVES * 64, true>(a.dst[0], a.dst[1], a.dst[2], b.kc, b.vc, b.part, b.done, b.out,
                                                                  b.H, b.L, b.pos, b.freq_scale, b.theta_scale, b.scale,
-                                                                 t % b.H, t / b.H, b.S, b.ready, b.target);
+                                                                 t % b.H, t / b.H, b.S, b.ready, b.target, b.key_stride,
+                                                                 b.head_stride);
     }
 }
 
 template <typename CT>
 int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, CT *k_cache, CT *v_cache, float *out,
                         int32_t n_head, int32_t head_dim, int32_t n_past, const int32_t *pos, float freq_scale,
-                        float theta_scale, float scale, const char *what) {
+                        float theta_scale, float scale, int32_t head_major_n_ctx, const char *what) {
     GH_REQUIRE_CTX(ctx);
     GH_REQUIRE(ctx, items && k_cache && v_cache && out && pos, GALOIS_HIP_E_NULL, what);
     GH_REQUIRE(ctx, head_dim == FA_HEAD_DIM, GALOIS_HIP_E_UNSUPPORTED, "qkv_attn_decode: head_dim 128");
+    GH_REQUIRE(ctx, head_major_n_ctx == 0 || head_major_n_ctx > n_past, GALOIS_HIP_E_SHAPE,
+               "qkv_attn_decode: head_major_n_ctx is 0 or the capacity of a [n_head][n_ctx][head_dim] cache, above n_past");
     GH_REQUIRE(ctx, n_head > 0 && n_head <= GH_ATTN_HEADS && n_past >= 0 && n_past < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
                "qkv_attn_decode: n_head in 1..65536, n_past >= 0");
     GH_REQUIRE(ctx, gh_aligned(k_cache, 16) && gh_aligned(v_cache, 16) && gh_aligned(out, 16) && gh_aligned(pos, 4),
@@ -942,6 +946,8 @@ int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, 
     b.H = n_head, b.L = L, b.S = S, b.gemv_blocks = (int32_t)plan.blocks;
     b.target = FA_HEAD_DIM / (FA_WAVES * FA_R);  // product workgroups per head
     b.freq_scale = freq_scale, b.theta_scale = theta_scale, b.scale = scale;
+    b.key_stride = head_major_n_ctx ? head_dim : (int64_t)n_head * head_dim;
+    b.head_stride = head_major_n_ctx ? (int64_t)head_major_n_ctx * head_dim : head_dim;
     GH_BIND(ctx);
     const dim3 grid((unsigned)(plan.blocks + (int64_t)n_head * S)), block(FA_WAVES * 64);
     size_t lds = (size_t)plan.max_slots * slot_lds<5>::bytes_per_slot;
@@ -1001,15 +1007,15 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *
 extern "C" int32_t galois_hip_qkv_attn_decode_f32(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, float *k_cache,
                                                   float *v_cache, float *out, int32_t n_head, int32_t head_dim,
                                                   int32_t n_past, const int32_t *pos, float freq_scale, float theta_scale,
-                                                  float scale) {
+                                                  float scale, int32_t head_major_n_ctx) {
     return launch_qkv_attn<float>(ctx, qkv, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
-                                  scale, "qkv_attn_decode_f32");
+                                  scale, head_major_n_ctx, "qkv_attn_decode_f32");
 }
 
 extern "C" int32_t galois_hip_qkv_attn_decode_f16kv(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, void *k_cache,
                                                     void *v_cache, float *out, int32_t n_head, int32_t head_dim,
                                                     int32_t n_past, const int32_t *pos, float freq_scale,
-                                                    float theta_scale, float scale) {
+                                                    float theta_scale, float scale, int32_t head_major_n_ctx) {
     return launch_qkv_attn<_Float16>(ctx, qkv, (_Float16 *)k_cache, (_Float16 *)v_cache, out, n_head, head_dim, n_past, pos,
-                                     freq_scale, theta_scale, scale, "qkv_attn_decode_f16kv");
+                                     freq_scale, theta_scale, scale, head_major_n_ctx, "qkv_attn_decode_f16kv");
 }

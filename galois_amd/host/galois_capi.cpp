@@ -156,12 +156,12 @@ void *galois_host_llama_new(void *dev, size_t n_vocab, size_t n_embd, size_t n_h
     }
     return m.release();
 }
-// the same with the KV cache in f16 when kv_f16 is non-zero
+// the same with a choice of KV cache: bit 0 of kv_flags = f16, bit 1 = kept head-major
 void *galois_host_llama_new_kv(void *dev, size_t n_vocab, size_t n_embd, size_t n_head, size_t n_layer, size_t n_ff,
-                               size_t n_ctx, float rms_eps, float freq_base, int kv_f16) {
+                               size_t n_ctx, float rms_eps, float freq_base, int kv_flags) {
     LlamaHParams hp;
     hp.n_vocab = n_vocab, hp.n_embd = n_embd, hp.n_head = n_head, hp.n_layer = n_layer, hp.n_ff = n_ff, hp.n_ctx = n_ctx;
-    hp.rms_eps = rms_eps, hp.freq_base = freq_base, hp.kv_f16 = kv_f16 != 0;
+    hp.rms_eps = rms_eps, hp.freq_base = freq_base, hp.kv_f16 = (kv_flags & 1) != 0, hp.kv_head_major = (kv_flags & 2) != 0;
     std::unique_ptr<LlamaDecoder> m;
     GResult r = LlamaDecoder::create(hp, *(Device *)dev, &m);
     if (!r.ok()) {

@@ -91,9 +91,10 @@ GResult galois_matvec_group(const std::vector<MatvecItem> &items) {
 }
 
 // The checks both attention calls share; dev receives the tensors' device.
+// head_major_n_ctx receives 0 for caches [n_embd, n_ctx] and n_ctx for caches [head_dim, n_ctx, n_head].
 static GResult attn_check(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                           Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past,
-                          std::shared_ptr<CudaDevice> &dev) {
+                          std::shared_ptr<CudaDevice> &dev, int32_t *head_major_n_ctx) {
     for (const Tensor *t : {&q, &k, &v, (const Tensor *)&k_cache, (const Tensor *)&v_cache, &pos, (const Tensor *)&out}) {
         if (!t->device().is_gpu()) return err(GError::Unimplemented, "galois_attn_decode: Gpu tensors only");
         if (!dev) dev = t->device().gpu;
@@ -107,26 +108,35 @@ static GResult attn_check(const RopeCustomOption &op, const Tensor &q, const Ten
     if (op.mode != 0) return err(GError::Unimplemented, "galois_attn_decode: rope mode 0 only (src/cuda.rs:1336-1340)");
     const size_t E = q.dim().elem_count();
     if (n_head == 0 || E % n_head != 0 || op.n_dims != E / n_head || k.dim().elem_count() != E || v.dim().elem_count() != E ||
-        out.dim().elem_count() != E || k_cache.dim().shape[0] != E || v_cache.dim().shape[0] != E || pos.dim().elem_count() != 1 ||
-        n_past < 0 || (size_t)n_past >= k_cache.dim().shape[1] || (size_t)n_past >= v_cache.dim().shape[1])
-        return err(GError::ShapeError, "galois_attn_decode: q, k, v, out of n_head * n_dims elements, caches [that, n_ctx], n_past < n_ctx");
+        out.dim().elem_count() != E || pos.dim().elem_count() != 1 || n_past < 0 || (size_t)n_past >= k_cache.dim().shape[1] ||
+        (size_t)n_past >= v_cache.dim().shape[1])
+        return err(GError::ShapeError, "galois_attn_decode: q, k, v, out of n_head * n_dims elements, n_past < n_ctx");
+    const bool head_major = k_cache.dim().n_dims == 3;
+    for (const Tensor *c : {(const Tensor *)&k_cache, (const Tensor *)&v_cache}) {
+        const Dim &d = c->dim();
+        const bool ok = head_major ? (d.n_dims == 3 && d.shape[0] == E / n_head && d.shape[2] == n_head && d.shape[1] == k_cache.dim().shape[1])
+                                   : (d.n_dims == 2 && d.shape[0] == E);
+        if (!ok) return err(GError::ShapeError, "galois_attn_decode: both caches [n_embd, n_ctx] or both [head_dim, n_ctx, n_head]");
+    }
+    *head_major_n_ctx = head_major ? (int32_t)k_cache.dim().shape[1] : 0;
     return GError{};
 }
 
 GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                            Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale) {
     std::shared_ptr<CudaDevice> dev;
-    G_TRY(attn_check(op, q, k, v, k_cache, v_cache, pos, out, n_head, n_past, dev));
+    int32_t hm = 0;
+    G_TRY(attn_check(op, q, k, v, k_cache, v_cache, pos, out, n_head, n_past, dev, &hm));
     const size_t E = q.dim().elem_count();
     const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);  // as galois_rope_custom derives it (src/cuda.rs:1327)
     if (k_cache.dtype() == GGmlType::F16)
         return dev->check(galois_hip_attn_decode_f16kv(dev->ctx(), (const float *)q.data(), (const float *)k.data(),
                                                        (const float *)v.data(), k_cache.data(), v_cache.data(), (float *)out.data(),
                                                        (int32_t)n_head, (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(),
-                                                       op.freq_scale, theta_scale, scale));
+                                                       op.freq_scale, theta_scale, scale, hm));
     return dev->check(galois_hip_attn_decode_f32(dev->ctx(), (const float *)q.data(), (const float *)k.data(), (const float *)v.data(),
                                                  (float *)k_cache.data(), (float *)v_cache.data(), (float *)out.data(), (int32_t)n_head,
-                                                 (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
+                                                 (int32_t)(E / n_head), n_past, (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale, hm));
 }
 
 GResult galois_qkv_attn_decode(const RopeCustomOption &op, const std::vector<MatvecItem> &qkv, Tensor &k_cache, Tensor &v_cache,
@@ -135,17 +145,18 @@ GResult galois_qkv_attn_decode(const RopeCustomOption &op, const std::vector<Mat
     galois_hip_gemv_item it[8];
     std::shared_ptr<CudaDevice> dev, adev;
     G_TRY(matvec_items(qkv, it, dev));
-    G_TRY(attn_check(op, *qkv[0].dst, *qkv[1].dst, *qkv[2].dst, k_cache, v_cache, pos, out, n_head, n_past, adev));
+    int32_t hm = 0;
+    G_TRY(attn_check(op, *qkv[0].dst, *qkv[1].dst, *qkv[2].dst, k_cache, v_cache, pos, out, n_head, n_past, adev, &hm));
     if (adev != dev) return err(GError::Unimplemented, "galois_qkv_attn_decode: one device");
     const size_t E = out.dim().elem_count();
     const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);
     if (k_cache.dtype() == GGmlType::F16)
         return dev->check(galois_hip_qkv_attn_decode_f16kv(dev->ctx(), it, k_cache.data(), v_cache.data(), (float *)out.data(),
                                                            (int32_t)n_head, (int32_t)(E / n_head), n_past,
-                                                           (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
+                                                           (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale, hm));
     return dev->check(galois_hip_qkv_attn_decode_f32(dev->ctx(), it, (float *)k_cache.data(), (float *)v_cache.data(),
                                                      (float *)out.data(), (int32_t)n_head, (int32_t)(E / n_head), n_past,
-                                                     (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale));
+                                                     (const int32_t *)pos.data(), op.freq_scale, theta_scale, scale, hm));
 }
 
 static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t ne1 = 0, size_t ne2 = 0) {
@@ -177,8 +188,14 @@ GResult LlamaDecoder::create(const LlamaHParams &hp, const Device &dev, std::uni
         G_TRY(mk(&l.w_gate, Q, dev, E, F));
         G_TRY(mk(&l.w_up, Q, dev, E, F));
         G_TRY(mk(&l.w_down, Q, dev, F, E));
-        G_TRY(mk(&l.k_cache, hp.kv_f16 ? GGmlType::F16 : F32, dev, E, C));
-        G_TRY(mk(&l.v_cache, hp.kv_f16 ? GGmlType::F16 : F32, dev, E, C));
+        const GGmlType ct = hp.kv_f16 ? GGmlType::F16 : F32;
+        if (hp.kv_head_major) {
+            G_TRY(mk(&l.k_cache, ct, dev, D, C, H));
+            G_TRY(mk(&l.v_cache, ct, dev, D, C, H));
+        } else {
+            G_TRY(mk(&l.k_cache, ct, dev, E, C));
+            G_TRY(mk(&l.v_cache, ct, dev, E, C));
+        }
     }
     G_TRY(mk(&m->tok_id_, GGmlType::I32, dev, 1));
     G_TRY(mk(&m->pos_, GGmlType::I32, dev, 1));
@@ -321,23 +338,36 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
         G_TRY(k_.view(0, 3, hs, &kv));
         G_TRY(galois_rope_custom(rope, qv, pos_, qr_));
         G_TRY(galois_rope_custom(rope, kv, pos_, kr_)); ops += 2;
-        // append this position to the cache
+        // append this position to the cache: row n_past of [n_ctx][E], or row n_past of every head of [H][n_ctx][D]
         const size_t row[2] = {E, 1};
-        G_TRY(l.k_cache.view((size_t)n_past * E, 2, row, &k_row));
-        G_TRY(l.v_cache.view((size_t)n_past * E, 2, row, &v_row));
-        Tensor kr_flat;
-        G_TRY(kr_.view(0, 2, row, &kr_flat));
-        G_TRY(galois_cpy(kr_flat, k_row));
-        G_TRY(galois_cpy(v_, v_row)); ops += 2;
-        // scores = K^T q per head: K seen as [D, L, H] with strides (1, E, D)
+        const bool hm = hp_.kv_head_major;
+        if (hm) {
+            const size_t rsh[2] = {D, H}, rst[2] = {1, C * D};
+            G_TRY(l.k_cache.view_strided((size_t)n_past * D, 2, rsh, rst, &k_row));
+            G_TRY(l.v_cache.view_strided((size_t)n_past * D, 2, rsh, rst, &v_row));
+            Tensor kr2, v2;
+            G_TRY(kr_.view(0, 2, rsh, &kr2));
+            G_TRY(v_.view(0, 2, rsh, &v2));
+            G_TRY(galois_cpy(kr2, k_row));
+            G_TRY(galois_cpy(v2, v_row));
+        } else {
+            G_TRY(l.k_cache.view((size_t)n_past * E, 2, row, &k_row));
+            G_TRY(l.v_cache.view((size_t)n_past * E, 2, row, &v_row));
+            Tensor kr_flat;
+            G_TRY(kr_.view(0, 2, row, &kr_flat));
+            G_TRY(galois_cpy(kr_flat, k_row));
+            G_TRY(galois_cpy(v_, v_row));
+        }
+        ops += 2;
+        // scores = K^T q per head: K seen as [D, L, H] with strides (1, E, D), or (1, D, n_ctx * D) in a head-major cache
         Tensor kc, vc;
-        const size_t ksh[3] = {D, L, H}, kst[3] = {1, E, D};
+        const size_t ksh[3] = {D, L, H}, kst[3] = {1, hm ? D : E, hm ? C * D : D};
         G_TRY(l.k_cache.view_strided(0, 3, ksh, kst, &kc));
         G_TRY(galois_matmul(kc, q3, s));
         G_TRY(galois_scale(s, scale_, s));
         G_TRY(galois_soft_max(s, p)); ops += 3;
-        // out = V p per head: V seen as [L, D, H] with strides (E, 1, D)
-        const size_t vsh[3] = {L, D, H}, vst[3] = {E, 1, D};
+        // out = V p per head: V seen as [L, D, H] with strides (E, 1, D), or (D, 1, n_ctx * D)
+        const size_t vsh[3] = {L, D, H}, vst[3] = {hm ? D : E, 1, hm ? C * D : D};
         G_TRY(l.v_cache.view_strided(0, 3, vsh, vst, &vc));
         G_TRY(galois_matmul(vc, p, o_)); ops++;
         Tensor o_flat;

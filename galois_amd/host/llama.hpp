@@ -18,6 +18,7 @@ struct LlamaHParams {
     size_t n_vocab = 32000, n_embd = 4096, n_head = 32, n_layer = 32, n_ff = 11008, n_ctx = 2048;
     float rms_eps = 1e-6f, freq_base = 10000.0f, freq_scale = 1.0f;
     bool kv_f16 = false;  // KV cache in f16 (as the reference keeps it on the GPU); needs the fused attention (fused = 3)
+    bool kv_head_major = false;  // caches kept [head_dim, n_ctx, n_head] instead of [n_embd, n_ctx]: a head's keys contiguous
 };
 
 class LlamaDecoder {
@@ -29,7 +30,8 @@ class LlamaDecoder {
 
     // Weights by name: "tok_embd" [n_embd, n_vocab] Q4_0, "out_norm" [n_embd] F32, "output" [n_embd, n_vocab] Q4_0
     // (layer = -1), and per layer "attn_norm", "ffn_norm" F32, "wq", "wk", "wv", "wo" [n_embd, n_embd],
-    // "w_gate", "w_up" [n_embd, n_ff], "w_down" [n_ff, n_embd] Q4_0, "k_cache", "v_cache" [n_embd, n_ctx] F32.
+    // "w_gate", "w_up" [n_embd, n_ff], "w_down" [n_ff, n_embd] Q4_0, "k_cache", "v_cache" [n_embd, n_ctx] F32 or F16
+    // ([head_dim, n_ctx, n_head] with kv_head_major).
     Tensor *tensor(const std::string &name, int layer);
 
     // Enqueues one step for `token` at position n_past (attention over n_past + 1 keys); logits() holds the

@@ -226,13 +226,13 @@ class LlamaDecoder:
     """One-token decode step of a LLaMA-architecture model issued as galois ops (galois_amd/host/llama.hpp)."""
 
     def __init__(self, device, n_vocab=32000, n_embd=4096, n_head=32, n_layer=32, n_ff=11008, n_ctx=2048,
-                 rms_eps=1e-6, freq_base=10000.0, kv_f16=False, _handle=None):
+                 rms_eps=1e-6, freq_base=10000.0, kv_f16=False, kv_head_major=False, _handle=None):
         self.device = device
         self.hp = dict(n_vocab=n_vocab, n_embd=n_embd, n_head=n_head, n_layer=n_layer, n_ff=n_ff, n_ctx=n_ctx,
                        rms_eps=rms_eps, freq_base=freq_base)
-        self.kv_f16 = bool(kv_f16)
+        self.kv_f16, self.kv_head_major = bool(kv_f16), bool(kv_head_major)
         self.h = _handle or lib().galois_host_llama_new_kv(device.h, n_vocab, n_embd, n_head, n_layer, n_ff, n_ctx,
-                                                           rms_eps, freq_base, int(self.kv_f16))
+                                                           rms_eps, freq_base, int(self.kv_f16) | 2 * int(self.kv_head_major))
         if not self.h:
             _raise(3)
 
@@ -261,8 +261,9 @@ class LlamaDecoder:
         shapes = {"tok_embd": ((e, v), Q4_0), "output": ((e, v), Q4_0), "out_norm": ((e,), F32),
                   "attn_norm": ((e,), F32), "ffn_norm": ((e,), F32), "wq": ((e, e), Q4_0), "wk": ((e, e), Q4_0),
                   "wv": ((e, e), Q4_0), "wo": ((e, e), Q4_0), "w_gate": ((e, f), Q4_0), "w_up": ((e, f), Q4_0),
-                  "w_down": ((f, e), Q4_0), "k_cache": ((e, c), F16 if self.kv_f16 else F32),
-                  "v_cache": ((e, c), F16 if self.kv_f16 else F32)}
+                  "w_down": ((f, e), Q4_0)}
+        cache = (e // hp["n_head"], c, hp["n_head"]) if self.kv_head_major else (e, c)   # numpy sees [H, C, D] or [C, E]
+        shapes["k_cache"] = shapes["v_cache"] = (cache, F16 if self.kv_f16 else F32)
         shape, dtype = shapes[name]
         t = Tensor(h, shape, dtype)
         t.borrowed = True

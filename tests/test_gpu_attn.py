@@ -121,6 +121,46 @@ def test_attn_decode_with_f16_caches(dev, H, D, n_ctx, n_past):
         dev.free(b)
 
 
+@pytest.mark.parametrize("H,D,n_ctx,n_past,f16", [(32, 128, 2048, 2047, False), (32, 128, 2100, 130, False),
+                                                  (3, 64, 300, 299, False), (2, 128, 64, 0, False),
+                                                  (32, 128, 2048, 2047, True), (5, 64, 700, 640, True)])
+def test_head_major_caches_give_the_same_bits(dev, H, D, n_ctx, n_past, f16):
+    """Caches kept [n_head][n_ctx][head_dim] hold the same elements at other addresses: the output and the cache
+    contents equal those of the [n_ctx][n_head * head_dim] call bit for bit, for all three entry points."""
+    rng = np.random.default_rng(H + D + n_past)
+    E = H * D
+    ct = np.float16 if f16 else np.float32
+    q, k, v = (rng.standard_normal(E).astype(np.float32) for _ in range(3))
+    kc = rng.standard_normal((n_ctx, E)).astype(ct)
+    vc = rng.standard_normal((n_ctx, E)).astype(ct)
+    hm = lambda c: np.ascontiguousarray(c.reshape(n_ctx, H, D).transpose(1, 0, 2))       # [H][n_ctx][D]
+    fs, ts, scale = 1.0, float(np.float32(10000.0) ** np.float32(-2.0 / D)), 1.0 / np.sqrt(D)
+    qb, kb, vb, pos = dev.upload(q), dev.upload(k), dev.upload(v), dev.upload(np.array([n_past], np.int32))
+    calls = [dev.attn_decode_f16kv] if f16 else [dev.attn_decode_f32, dev.attn_decode_f32_static]
+    for call in calls:
+        res = []
+        for layout in (0, n_ctx):
+            kcb, vcb = dev.upload(hm(kc) if layout else kc), dev.upload(hm(vc) if layout else vc)
+            out = dev.upload(np.full(E + 16, 7.5, np.float32))
+            call(qb, kb, vb, kcb, vcb, out, H, D, n_past, pos, fs, ts, scale, layout)
+            o = dev.download(out, np.float32, E + 16)
+            kg, vg = dev.download(kcb, ct, (H, n_ctx, D) if layout else (n_ctx, E)), dev.download(vcb, ct, (H, n_ctx, D) if layout else (n_ctx, E))
+            if layout:
+                kg, vg = kg.transpose(1, 0, 2).reshape(n_ctx, E), vg.transpose(1, 0, 2).reshape(n_ctx, E)
+            res.append((o, kg, vg))
+            for b in (kcb, vcb, out):
+                dev.free(b)
+        for a, b in zip(*res):
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+        assert np.all(res[1][0][E:] == 7.5) and np.all(np.isfinite(res[1][0][:E]))
+    if n_past > 0:
+        with pytest.raises(GaloisHipError) as ei:   # the capacity must exceed n_past
+            calls[0](qb, kb, vb, qb, qb, qb, H, D, n_past, pos, fs, ts, scale, n_past)
+        assert ei.value.status == -2
+    for b in (qb, kb, vb, pos):
+        dev.free(b)
+
+
 def test_attn_decode_invariants(dev):
     """One key: the output is that key's value row whatever q is.  Equal keys: the mean of the values."""
     H, D, n_ctx = 4, 128, 512

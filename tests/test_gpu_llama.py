@@ -34,9 +34,12 @@ def _load(dec, w, kc=None, vc=None):
     for i, lw in enumerate(w["layers"]):
         for n, a in lw.items():
             dec.tensor(n, i).write(a)
-        if kc is not None:
-            dec.tensor("k_cache", i).write(kc[i])
-            dec.tensor("v_cache", i).write(vc[i])
+        if kc is not None:   # kc[i] is [n_ctx][n_embd]; a head-major decoder keeps [n_head][n_ctx][head_dim]
+            hm = getattr(dec, "kv_head_major", False)
+            h = dec.hp["n_head"]
+            lay = (lambda c: np.ascontiguousarray(c.reshape(c.shape[0], h, -1).transpose(1, 0, 2))) if hm else (lambda c: c)
+            dec.tensor("k_cache", i).write(lay(kc[i]))
+            dec.tensor("v_cache", i).write(lay(vc[i]))
 
 
 def _ref_step(w, hp, kc, vc, token, n_past, round_kv=False):
@@ -150,6 +153,35 @@ def test_decode_with_an_f16_kv_cache(gdev):
     dec.close()
 
 
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_decode_with_head_major_caches(gdev, kv_f16):
+    """Caches kept [n_head][n_ctx][head_dim]: every launch plan against the oracle on a filled cache (the plans built
+    from single ops reach the cache through strided views), the appended rows in their head-major places."""
+    rng = np.random.default_rng(57)
+    hp = SMALL
+    w = _make_weights(rng, hp)
+    n_past = 41
+    ct = np.float16 if kv_f16 else np.float32
+    kc = rng.standard_normal((hp["n_layer"], hp["n_ctx"], hp["n_embd"])).astype(ct)
+    vc = rng.standard_normal((hp["n_layer"], hp["n_ctx"], hp["n_embd"])).astype(ct)
+    dec = g.LlamaDecoder(gdev, kv_f16=kv_f16, kv_head_major=True, **hp)
+    kc_ref, vc_ref = kc.astype(np.float32), vc.astype(np.float32)
+    ref = _ref_step(w, hp, kc_ref, vc_ref, 77, n_past, round_kv=kv_f16)
+    for fused in ((3, 4, 5) if kv_f16 else (0, 1, 2, 3, 4, 5)):
+        _load(dec, w, kc, vc)
+        dec.decode(77, n_past, fused)
+        _check(dec.logits(), ref, 2e-4 if kv_f16 else 1e-4)
+    h, d = hp["n_head"], hp["n_embd"] // hp["n_head"]
+    for i in range(hp["n_layer"]):
+        kg = dec.tensor("k_cache", i).to_cpu_tensor()
+        assert kg.shape == (h, hp["n_ctx"], d) and kg.dtype == ct
+        kg = kg.transpose(1, 0, 2).reshape(hp["n_ctx"], -1)
+        rows = np.arange(hp["n_ctx"]) != n_past
+        assert np.array_equal(kg[rows], kc[i][rows])
+        _check(kg[n_past].astype(np.float32), kc_ref[i][n_past], 1e-3 if kv_f16 else 1e-4)
+    dec.close()
+
+
 def test_graph_replays_equal_the_eager_step(gdev):
     rng = np.random.default_rng(52)
     hp = SMALL
@@ -222,4 +254,11 @@ def test_full_width_layers_at_kv_length_2048(gdev):
         _load(dec, w, kc16, vc16)
         dec.decode(31999, 2047, fused)
         _check(dec.logits(), ref16, 2e-4)
+    dec.close()
+    # head-major f32 caches at full width: the two shortest plans
+    dec = g.LlamaDecoder(gdev, kv_head_major=True, **hp)
+    for fused in (4, 5):
+        _load(dec, w, kc, vc)
+        dec.decode(31999, 2047, fused)
+        _check(dec.logits(), ref, 1e-4)
     dec.close()

@@ -69,6 +69,40 @@ def test_qkv_attn_equals_the_two_calls(dev, H, K, n_past, mode, kv_f16):
     _case(dev, H, K, n_past, mode, kv_f16, seed=H * 1000 + n_past)
 
 
+@pytest.mark.parametrize("H,K,n_past,n_ctx,kv_f16", [(32, 4096, 2047, 2048, False), (3, 256, 130, 200, True)])
+def test_qkv_attn_with_head_major_caches(dev, H, K, n_past, n_ctx, kv_f16):
+    """The same launch over caches kept [n_head][n_ctx][head_dim]: outputs and cache contents bit-equal."""
+    D = 128
+    E = H * D
+    rng = np.random.default_rng(H + n_past)
+    ct = np.float16 if kv_f16 else np.float32
+    ws = [dev.upload(oracle.quantize_q4_0((rng.standard_normal((E, K)) * 0.05).astype(np.float32))) for _ in range(3)]
+    x, nw = dev.upload(rng.standard_normal(K).astype(np.float32)), dev.upload(np.ones(K, np.float32))
+    kc0, vc0 = rng.standard_normal((n_ctx, E)).astype(ct), rng.standard_normal((n_ctx, E)).astype(ct)
+    hm = lambda c: np.ascontiguousarray(c.reshape(n_ctx, H, D).transpose(1, 0, 2))
+    pos = dev.upload(np.array([n_past], np.int32))
+    res = []
+    for layout in (0, n_ctx):
+        q, k, v = (dev.alloc(E * 4) for _ in range(3))
+        items = dev.gemv_items([{"vx": w, "y": x, "dst": d, "ncols": K, "nrows": E, "norm_weight": nw, "norm_eps": 1e-5}
+                                for w, d in zip(ws, (q, k, v))])
+        kcb, vcb, out = dev.upload(hm(kc0) if layout else kc0), dev.upload(hm(vc0) if layout else vc0), dev.alloc(E * 4)
+        dev.qkv_attn_decode(items, kcb, vcb, out, H, D, n_past, pos, 1.0, 10000.0 ** (-2.0 / D), D ** -0.5, kv_f16=kv_f16,
+                            head_major_n_ctx=layout)
+        shape = (H, n_ctx, D) if layout else (n_ctx, E)
+        o, kg, vg = dev.download(out, np.float32, E), dev.download(kcb, ct, shape), dev.download(vcb, ct, shape)
+        if layout:
+            kg, vg = kg.transpose(1, 0, 2).reshape(n_ctx, E), vg.transpose(1, 0, 2).reshape(n_ctx, E)
+        res.append((o, kg, vg))
+        for b in (q, k, v, kcb, vcb, out):
+            dev.free(b)
+    for a, b in zip(*res):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    assert np.all(np.isfinite(res[1][0]))
+    for b in ws + [x, nw, pos]:
+        dev.free(b)
+
+
 def test_qkv_attn_argument_errors(dev):
     from galois_amd import GaloisHipError
     rng = np.random.default_rng(1)
