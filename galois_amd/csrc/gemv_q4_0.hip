@@ -888,6 +888,7 @@ struct fa_args {
 constexpr int FA_WAVES = 8, FA_HEAD_DIM = 128;
 constexpr int FA_R = 2;  // rows per wave of the products (measured: 4, which makes all products resident at once, 30.7 against 25.3 us)
 static_assert(FA_HEAD_DIM % (FA_WAVES * FA_R) == 0, "a product workgroup's rows belong to one head");
+constexpr int FA_MAX_SLOTS = 184;  // activation vectors of up to 11776 elements: 55,936 bytes of planes beside the attention's 8.9 KB
 
 template <int PG, int NORM_MODE, typename CT>
 __global__ __launch_bounds__(FA_WAVES * 64, 4) void qkv_attn_decode_fused(const gg_args a, const fa_args<CT> b) {
@@ -933,6 +934,8 @@ int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, 
     gg_plan plan;
     const int32_t st = prepare_group(ctx, items, 3, what, a, plan, FA_WAVES * FA_R);
     if (st != GALOIS_HIP_OK) return st;
+    // the attention's own LDS (9 KB) shares the 64 KB of a workgroup with the products' activation planes
+    GH_REQUIRE(ctx, plan.max_slots <= FA_MAX_SLOTS, GALOIS_HIP_E_SHAPE, "qkv_attn_decode: ncols at most 11776");
     const int L = n_past + 1;
     const int S = (L + AT_KEYS - 1) / AT_KEYS;
     GH_REQUIRE(ctx, S <= AT_MAX_SPLITS && (S == 1 || ((int64_t)n_head * S * (head_dim + 4) <= GH_PARTIAL_FLOATS)) &&

@@ -255,8 +255,9 @@ GResult LlamaDecoder::step(int32_t n_past, int fused) {
         return err(GError::Unimplemented, "LlamaDecoder: the grouped launch plans (fused >= 2) need n_embd and n_ff to be "
                                           "multiples of 64 no larger than 12288; use fused = 0 or 1");
     const size_t E = hp_.n_embd, H = hp_.n_head, D = E / H, L = (size_t)n_past + 1, C = hp_.n_ctx;
-    if (fused >= 5 && D != 128)
-        return err(GError::Unimplemented, "LlamaDecoder: the launch that carries q | k | v and the attention (fused = 5) needs heads of 128");
+    if (fused >= 5 && (D != 128 || E > 11776))
+        return err(GError::Unimplemented, "LlamaDecoder: the launch that carries q | k | v and the attention (fused = 5) needs heads of 128 "
+                                          "and n_embd up to 11776");
     RopeCustomOption rope;
     rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;
     size_t ops = 0;

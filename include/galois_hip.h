@@ -280,8 +280,9 @@ int32_t galois_hip_attn_decode_f16kv(galois_hip_ctx *ctx, const float *q, const 
  * The attention's workgroups follow the products' in the grid, request their cache rows while the last products
  * still stream, and wait -- bounded -- only for their own head's rows of q (k and v where position n_past lives);
  * should a wait ever run out, that head's output is NaN.  q, k, v and the appended cache rows equal those of the two
- * calls issued one after the other bit for bit, the output up to the order of its f32 sums.  head_dim 128; the products are plain or normalising (no vx_up, residual, dst_scaled, sumsq_out); dst
- * 16-byte aligned; limits of both calls apply. */
+ * calls issued one after the other bit for bit (when the group call would run few rows in its 16-wave shape: up to the
+ * order in which a normalising product adds its squares), the output up to the order of its f32 sums.  head_dim 128; the products are plain or normalising (no vx_up, residual, dst_scaled, sumsq_out); dst
+ * 16-byte aligned; ncols <= 11776; otherwise the limits of both calls apply. */
 int32_t galois_hip_qkv_attn_decode_f32(galois_hip_ctx *ctx, const galois_hip_gemv_item *qkv, float *k_cache,
                                        float *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
                                        const int32_t *pos, float freq_scale, float theta_scale, float scale, int32_t head_major_n_ctx);

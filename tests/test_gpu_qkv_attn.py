@@ -1,7 +1,9 @@
 """The launch that carries the q | k | v products and the decode attention together against the same two calls issued
-one after the other: q, k, v and the appended cache rows are bit-equal; the attention's output agrees up to the order
-of its f32 sums (eight waves instead of four share a split's keys): 1e-5 of the largest output, the tolerance of the
-attention's own parity test."""
+one after the other.  q, k, v and the appended cache rows are bit-equal whenever the products' own call runs the same
+workgroup shape (8 waves x 2 rows); with few rows it runs 16 waves x 1 row, which adds up a normalising product's
+sum of squares in another order, so there the bar is 2e-6 of the largest element.  The attention's output agrees up to
+the order of its f32 sums (eight waves instead of four share a split's keys): 1e-5 of the largest output, the
+tolerance of the attention's own parity test."""
 import numpy as np
 import pytest
 
@@ -52,8 +54,11 @@ def _case(dev, H, K, n_past, mode, kv_f16, seed, repeats=1, n_ctx=None):
             if name == "out":
                 assert np.all(np.isfinite(rb[:E])) and np.all(rb[E:] == 7.5)
                 assert np.max(np.abs(ra[:E] - rb[:E])) <= 1e-5 * np.max(np.abs(ra[:E])), r
-            else:
+            elif 3 * E > 16 * 256:   # more than 16 rows per CU: the products' own call runs the same workgroup shape
                 assert np.array_equal(ra.view(np.uint8), rb.view(np.uint8)), (name, r)
+            else:
+                fa, fb = ra.astype(np.float32), rb.astype(np.float32)
+                assert np.max(np.abs(fa - fb)) <= (1e-3 if kv_f16 else 2e-6) * np.max(np.abs(fa)), (name, r)
     for s in (a, b):
         for key in ("q", "k", "v", "kc", "vc", "out"):
             dev.free(s[key])
@@ -63,7 +68,7 @@ def _case(dev, H, K, n_past, mode, kv_f16, seed, repeats=1, n_ctx=None):
 
 @pytest.mark.parametrize("H,K,n_past,mode,kv_f16", [
     (2, 256, 0, 0, False), (2, 256, 5, 1, False), (3, 320, 130, 2, False), (4, 256, 127, 1, True),
-    (2, 5120, 300, 1, False), (2, 4160, 300, 2, True), (2, 4160, 40, 0, False),
+    (2, 5120, 300, 1, False), (2, 4160, 300, 2, True), (2, 4160, 40, 0, False), (2, 11776, 70, 1, False),
     (32, 4096, 2047, 2, False), (32, 4096, 2047, 1, False), (32, 4096, 2047, 2, True), (32, 4096, 2300, 0, False)])
 def test_qkv_attn_equals_the_two_calls(dev, H, K, n_past, mode, kv_f16):
     _case(dev, H, K, n_past, mode, kv_f16, seed=H * 1000 + n_past)
@@ -116,7 +121,8 @@ def test_qkv_attn_argument_errors(dev):
     for items, h, d, code in ((ok, H, 64, -5),                                           # heads of 128 only
                               ([item, item, dict(item, nrows=E - 16)], H, D, -2),        # every product n_head * head_dim rows
                               ([item, item, dict(item, residual=x)], H, D, -5),          # no residual, pair or second output
-                              (ok, 0, D, -2)):
+                              (ok, 0, D, -2),
+                              ([dict(item, ncols=12288)] * 3, H, D, -2)):                # vectors of up to 11776
         with pytest.raises(GaloisHipError) as ei:
             dev.qkv_attn_decode(items, kc, kc, out, h, d, 0, pos, 1.0, 0.9, 0.1)
         assert ei.value.status == code, (ei.value.status, code)
