@@ -87,6 +87,22 @@ def test_gemm_prefill_config(dev):
         dev.free(b)
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 4096, 4096), (512, 11008, 4096), (512, 4096, 4112), (256, 4096, 8192)])
+def test_gemm_narrow_matrices_at_full_size(dev, m, k, n):
+    """The other prefill products of a LLaMA-7B layer (N = 4096), which run the narrower column tile (48 columns per
+    workgroup instead of 96, chosen by how many workgroups that gives the device), and two more sizes: a column
+    sample against the oracle and linearity at the full size."""
+    wq, x = _case(m + k + n, m, k, n)
+    got = _gemm(dev, wq, x)
+    cols = np.random.default_rng(5).choice(n, 192, replace=False)
+    cols[:3] = (0, n - 1, n // 2)
+    emax, el2 = npref.rel_err(got[:, cols], oracle.mul_mat_q4_0_f32(wq[cols], x))
+    assert emax < TOL and el2 < TOL, (emax, el2)
+    got2 = _gemm(dev, wq, (0.5 * x).astype(np.float32))
+    emax, el2 = npref.rel_err(got2, 0.5 * got)
+    assert emax < 1e-6 and el2 < 1e-6
+
+
 def test_gemm_argument_errors(dev):
     from galois_amd import GaloisHipError
     buf = dev.alloc(4096)
