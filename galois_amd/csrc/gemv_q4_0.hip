@@ -407,8 +407,16 @@ struct gg_args {
 // MAXI: products the selects look at (4 keeps all of their operands in scalar registers at once).
 // COHERENT: the results go out as device-coherent stores, for readers in the same launch on other XCDs.
 // item / item_block: which product the workgroup served and its index among that product's workgroups.
-template <int L, int R, int WAVES, int PG, int NORM_MODE, int MAXI, bool OUT2, bool COHERENT>
+// CHUNKED: a vector longer than THREADS * PG / 8 slots is worked through in chunks of that many slots -- prepare a
+// chunk, meet, multiply it, meet, prepare the next -- so that the kernel keeps the registers and the LDS of the
+// short-vector build whatever the longest vector of the launch: measured on the four LLaMA-7B products in one
+// launch, the one K = 11008 matrix made all 3200 workgroups run the build that holds three tasks per thread and
+// 52 KB of planes (three workgroups per CU instead of four), 24.4 us against 23.1 us for the same bytes at K = 4096.
+// Not for the normalising preparation, which needs the whole vector's sum of squares before it scales anything.
+template <int L, int R, int WAVES, int PG, int NORM_MODE, int MAXI, bool OUT2, bool COHERENT, bool CHUNKED = false>
 __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, int &item, int &item_block) {
+    static_assert(!(CHUNKED && NORM_MODE == 1), "the normalising preparation is not chunked");
+    constexpr int CH = WAVES * 64 * PG / 8;  // slots per chunk
     __shared__ float red[WAVES];
     __shared__ float red2[WAVES];
     constexpr int SD = slot_lds<L>::dwords;
@@ -417,7 +425,9 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
     constexpr bool NORM2 = NORM_MODE == 2;   // scale the result by inv from the partial sums of squares
     constexpr bool NARG = NORM_MODE != 0;    // the norm_w / eps arguments are used
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // CHUNKED: the wave index as a scalar, so that row addresses are scalar too and do not hold vector registers
+    // through every phase of every chunk
+    const int wave = CHUNKED ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) : (int)(threadIdx.x >> 6);
 
     // Every product's fields are fetched before any is chosen (the empty asm makes each an opaque value; left
     // alone, the compiler turns a select of two arguments into a second, dependent load from a selected address).
@@ -459,13 +469,13 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
     typedef const __attribute__((address_space(1))) uint8_t *global_bytes;
     typedef const __attribute__((address_space(1))) float *global_floats;
     const uint8_t *const W = (const uint8_t *)(global_bytes)W_bits, *const W2 = (const uint8_t *)(global_bytes)W2_bits;
-    const float *const xg = (const float *)(global_floats)x_bits;
+    const float *const xg_all = (const float *)(global_floats)x_bits;
     item = ii, item_block = (int)blockIdx.x - first_blk;
     const bool dual = W2 != nullptr;
     const int rw = dual ? R / 2 : R;  // rows per wave and group
     // the workgroup's waves cover WAVES * rw consecutive rows: neighbouring waves read neighbouring rows
     const int row0 = ((int)blockIdx.x - first_blk) * (WAVES * rw) + wave * rw;
-    const size_t row_bytes = (size_t)ns * sizeof(q4_slot);
+    const size_t row_bytes = (size_t)ns * sizeof(q4_slot);  // of the whole row
 
     float acc[R];
 #pragma unroll
@@ -475,8 +485,28 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
     // are requested first and the first weights right behind them: the preparation then runs while the weights
     // are in flight.
     q4_slot q0[R];
-    uint64_t dst_bits, res_bits, dst2_bits = 0, scale2_bits = 0, ssq_bits = 0;
+    uint64_t dst_bits = 0, res_bits = 0, dst2_bits = 0, scale2_bits = 0, ssq_bits = 0;
     float scale2_first = 0.0f;  // OUT2: scale_weight of this lane's row
+    float inv2 = 1.0f;
+    const int ns_all = ns;  // the row's slots; below, ns is the chunk's
+    const int nchunks = CHUNKED ? (ns_all + CH - 1) / CH : 1;
+    constexpr int MAX_CHUNKS = CHUNKED ? (GG_MAX_SLOTS + CH - 1) / CH : 1;
+    // unrolled: as a loop the compiler hoists the chunk-independent address arithmetic into registers that then live
+    // through every phase (76 registers instead of 59)
+#pragma unroll
+    for (int chunk = 0; chunk < MAX_CHUNKS; chunk++) {
+    if (CHUNKED && chunk >= nchunks) break;
+    if (CHUNKED && chunk > 0) __builtin_amdgcn_sched_barrier(0);  // the next chunk's requests stay behind this point: their
+                                                                  // registers are not free before the multiplication is done
+    const int c0 = CHUNKED ? chunk * CH : 0;                     // first slot of the chunk
+    const int ns = CHUNKED ? min(CH, ns_all - c0) : ns_all;      // slots in it
+    const float *const xg = xg_all + (size_t)c0 * 64;
+    const bool first = !CHUNKED || chunk == 0;
+    // CHUNKED: the thread index passes through an empty asm in every chunk, so that what is derived from it (addresses in
+    // the vector, in LDS, in the row) is computed where it is used instead of living in registers from chunk to chunk
+    int tid_c = (int)threadIdx.x;
+    if (CHUNKED) asm volatile("" : "+v"(tid_c));
+    const int lane = tid_c & 63;
     {
         const float *wg = NORM ? (const float *)(global_floats)nw_bits : nullptr;
         float2 v[PG][4], nw[NORM ? PG : 1][4];
@@ -490,28 +520,28 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
         if (STAGED) {
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const int i4 = min((int)threadIdx.x + j * THREADS, ns * 16 - 1);
+                const int i4 = min(tid_c + j * THREADS, ns * 16 - 1);
                 sx[j] = reinterpret_cast<const float4 *>(xg)[i4];
                 sg[j] = reinterpret_cast<const float4 *>(wg)[i4];
             }
         }
 #pragma unroll
         for (int p = 0; p < PG; p++) {
-            const int idx = threadIdx.x + p * THREADS;
+            const int idx = tid_c + p * THREADS;
             if (!STAGED && idx < ns * 8) {
                 fetch_task(xg + (idx >> 3) * 64, idx & 7, v[p]);
                 if (NORM) fetch_task(wg + (idx >> 3) * 64, idx & 7, nw[NORM ? p : 0]);
             }
         }
         float psq = 0.0f;
-        if (NORM2) {  // one partial per 16 elements of the vector: ns * 4 of them
+        if (NORM2 && first) {  // one partial per 16 elements of the whole vector: ns_all * 4 of them
             const float *sq = (const float *)(global_floats)nw_bits;
             constexpr int PQ = (GG_MAX_SLOTS * 4 + THREADS - 1) / THREADS;
             float t[PQ];
 #pragma unroll
-            for (int p = 0; p < PQ; p++) t[p] = sq[min((int)threadIdx.x + p * THREADS, ns * 4 - 1)];
+            for (int p = 0; p < PQ; p++) t[p] = sq[min(tid_c + p * THREADS, ns_all * 4 - 1)];
 #pragma unroll
-            for (int p = 0; p < PQ; p++) psq += (int)threadIdx.x + p * THREADS < ns * 4 ? t[p] : 0.0f;
+            for (int p = 0; p < PQ; p++) psq += tid_c + p * THREADS < ns_all * 4 ? t[p] : 0.0f;
         }
         // q[j] = slot `lane` of row row0 + j of W; for a gate / up pair q[j] = row row0 + j of W (j < R/2) or of W2.
         // Rows past N are loaded from row N - 1 and never stored.
@@ -521,22 +551,24 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
             for (int j = 0; j < R; j++) {
                 const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
                 const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
-                load_slot(q0[j], base + (size_t)row * row_bytes + (size_t)s * sizeof(q4_slot));
+                load_slot(q0[j], base + (size_t)row * row_bytes + (size_t)(c0 + s) * sizeof(q4_slot));
             }
         }
         // nothing that waits for the activations may be scheduled ahead of the weight requests
         __builtin_amdgcn_sched_barrier(0);
         // Where the results go, fetched now (indexed argument loads) so that nothing waits for them at the end.
-        dst_bits = (uint64_t)a.dst[ii], res_bits = (uint64_t)a.residual[ii];
-        asm volatile("" : "+s"(dst_bits));
-        asm volatile("" : "+s"(res_bits));
-        if (OUT2) {
-            dst2_bits = (uint64_t)a.dst2[ii], scale2_bits = (uint64_t)a.scale2[ii], ssq_bits = (uint64_t)a.ssq_out[ii];
-            asm volatile("" : "+s"(dst2_bits));
-            asm volatile("" : "+s"(scale2_bits));
-            asm volatile("" : "+s"(ssq_bits));
+        if (first) {
+            dst_bits = (uint64_t)a.dst[ii], res_bits = (uint64_t)a.residual[ii];
+            asm volatile("" : "+s"(dst_bits));
+            asm volatile("" : "+s"(res_bits));
+            if (OUT2) {
+                dst2_bits = (uint64_t)a.dst2[ii], scale2_bits = (uint64_t)a.scale2[ii], ssq_bits = (uint64_t)a.ssq_out[ii];
+                asm volatile("" : "+s"(dst2_bits));
+                asm volatile("" : "+s"(scale2_bits));
+                asm volatile("" : "+s"(ssq_bits));
+            }
         }
-        if (NORM2) {  // the partial sums reach every wave through the barrier that publishes the planes
+        if (NORM2 && first) {  // the partial sums reach every wave through the barrier that publishes the planes
             psq = wave_sum(psq);
             if (lane == 0) red[wave] = psq;
         }
@@ -547,7 +579,7 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
             if (STAGED) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    const int i4 = (int)threadIdx.x + j * THREADS;
+                    const int i4 = tid_c + j * THREADS;
                     if (i4 < ns * 16) {
                         ss += sx[j].x * sx[j].x + sx[j].y * sx[j].y + sx[j].z * sx[j].z + sx[j].w * sx[j].w;
                         reinterpret_cast<float4 *>(stage)[i4] =
@@ -557,7 +589,7 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
             } else {
 #pragma unroll
                 for (int p = 0; p < PG; p++)
-                    if (threadIdx.x + p * THREADS < ns * 8) {
+                    if (tid_c + p * THREADS < ns * 8) {
 #pragma unroll
                         for (int t = 0; t < 4; t++) ss += v[p][t].x * v[p][t].x + v[p][t].y * v[p][t].y;
                     }
@@ -570,8 +602,8 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
             for (int w = 0; w < WAVES; w++) tot += red[w];
             const float inv = rsqrtf(tot / (float)(ns * 64) + eps);
             if (STAGED) {
-                if ((int)threadIdx.x < ns * 8) {
-                    fetch_task(stage + (threadIdx.x >> 3) * 64, threadIdx.x & 7, v[0]);
+                if (tid_c < ns * 8) {
+                    fetch_task(stage + (tid_c >> 3) * 64, tid_c & 7, v[0]);
 #pragma unroll
                     for (int t = 0; t < 4; t++) v[0][t] = make_float2(v[0][t].x * inv, v[0][t].y * inv);
                 }
@@ -590,7 +622,7 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
         uint32_t *const corr = lds + ns * SD + (STAGED ? ns * 64 : 0);
 #pragma unroll
         for (int p = 0; p < PG; p++) {
-            const int idx = threadIdx.x + p * THREADS;
+            const int idx = tid_c + p * THREADS;
             if (idx < ns * 8) {
                 const int slot = idx >> 3, g = idx & 7;
                 const float x8[8] = GH_TASK_X8(v[p]);
@@ -619,23 +651,24 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
         }
     }
     __syncthreads();
-    if (OUT2) {  // the scale values ride behind the weights, requested once the preparation's registers are free
+    if (OUT2 && first) {  // the scale values ride behind the weights, requested once the preparation's registers are free
         const float *sp = scale2_bits ? (const float *)(global_floats)scale2_bits + min(row0 + (lane < rw ? lane : 0), N - 1) : xg;
         scale2_first = *sp;
     }
-    float inv2 = 1.0f;
-    if (NORM2) {
+    if (NORM2 && first) {
         float tot = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; w++) tot += red[w];
         // the same value in every lane: kept in a scalar register (the kernel has no vector register to spare)
-        inv2 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrtf(tot / (float)(ns * 64) + eps))));
+        inv2 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrtf(tot / (float)(ns_all * 64) + eps))));
     }
-    float sq_out = 0.0f;  // OUT2: squares of this lane's results
 
     // The rows of this wave.  The first slots are the ones requested before the preparation.
     {
         const uint32_t *corr = lds + ns * SD + ((NORM && PG == 1) ? ns * 64 : 0);
+        if (CHUNKED) {  // a chunk is at most one slot per lane: the one requested before its preparation
+            if (lane < ns) slot_rows<L, R>(q0, lds + lane * SD, corr + lane * slot_lds<L>::corr_dwords, acc);
+        } else
         for (int sl = lane; sl - lane < ns; sl += 64) {  // uniform trip count; lanes past the end idle
             const bool act = sl < ns;
             const int s_ld = min(sl, ns - 1);
@@ -648,12 +681,17 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
                 for (int j = 0; j < R; j++) {
                     const uint8_t *base = (dual && j >= R / 2) ? W2 : W;
                     const int row = min(row0 + ((dual && j >= R / 2) ? j - R / 2 : j), N - 1);
-                    load_slot(q[j], base + (size_t)row * row_bytes + (size_t)s_ld * sizeof(q4_slot));
+                    load_slot(q[j], base + (size_t)row * row_bytes + (size_t)(c0 + s_ld) * sizeof(q4_slot));
                 }
             }
             if (act) slot_rows<L, R>(q, lds + s_ld * SD, corr + s_ld * slot_lds<L>::corr_dwords, acc);
         }
+    }
+    if (CHUNKED && chunk + 1 < nchunks) __syncthreads();  // every wave is done with this chunk's planes
+    }  // chunks
 
+    float sq_out = 0.0f;  // OUT2: squares of this lane's results
+    {
         // every total lands in lane 63; lane j picks up row j so the wave stores its rows at once
         float out = 0.0f;
         if (dual) {
@@ -703,11 +741,11 @@ __device__ __forceinline__ void gemv_group_wg(const gg_args &a, uint32_t *lds, i
     }
 }
 
-template <int L, int R, int WAVES, int PG, int OCC, int NORM_MODE, int MAXI, bool OUT2>
+template <int L, int R, int WAVES, int PG, int OCC, int NORM_MODE, int MAXI, bool OUT2, bool CHUNKED = false>
 __global__ __launch_bounds__(WAVES * 64, OCC) void gemv_q4_0_group(const gg_args a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     int item, item_block;
-    gemv_group_wg<L, R, WAVES, PG, NORM_MODE, MAXI, OUT2, false>(a, lds, item, item_block);
+    gemv_group_wg<L, R, WAVES, PG, NORM_MODE, MAXI, OUT2, false, CHUNKED>(a, lds, item, item_block);
 }
 
 template <int L, int R, int G, int WAVES, int OCC>
@@ -753,6 +791,20 @@ void launch_group_cfg(galois_hip_ctx *ctx, const gg_args &a, unsigned blocks, in
             GG_LAUNCH(PGSMALL, OCC, 0, (MAXI == 4), lds);
         else
             GG_LAUNCH(PGSMALL, OCC, 0, false, lds);
+    } else if (WAVES == 8 && mode != 1) {
+        // many rows and a long vector somewhere in the launch: chunks of 64 slots, so that every workgroup keeps the
+        // registers and the LDS of the short-vector build
+        const size_t lds_chunk = (size_t)64 * slot_lds<L>::bytes_per_slot;
+#define GG_LAUNCH_CHUNKED(MODE_, OUT2_)                                                                                \
+    hipLaunchKernelGGL((gemv_q4_0_group<L, R, WAVES, PGSMALL, OCC, MODE_, MAXI, OUT2_, true>), grid, block, lds_chunk, \
+                       ctx->stream, a)
+        if (mode == 2)
+            GG_LAUNCH_CHUNKED(2, false);
+        else if (out2 && MAXI == 4)
+            GG_LAUNCH_CHUNKED(0, (MAXI == 4));
+        else
+            GG_LAUNCH_CHUNKED(0, false);
+#undef GG_LAUNCH_CHUNKED
     } else {
         if (mode == 1)
             GG_LAUNCH(PGMAX, OCCN, 1, false, lds);

@@ -103,6 +103,30 @@ def test_group_llama7b_set_in_one_launch(dev):
         _check(got, oracle.mul_mat_q4_0_f32(it["vx"], it["y"]), it["vx"].shape)
 
 
+@pytest.mark.parametrize("k,n", [(4160, 4200), (8192, 4100), (11008, 4113), (12288, 4096), (4224, 9000)])
+def test_group_long_vectors_with_many_rows_in_chunks(dev, k, n):
+    """More than 16 rows per CU and a vector longer than 4096: the workgroups take the vector in chunks of 64 slots
+    (one slot in the last chunk, whole chunks, a ragged one).  Against the oracle, and bit-equal to the one-product
+    entry point; beside a short-vector product in the same launch; with activations whose blocks need correction
+    planes in every chunk."""
+    rng = np.random.default_rng(k + n)
+    wq = _wx(k * 3 + n, k, n)
+    x = rng.standard_normal(k).astype(np.float32)
+    xh = x.copy()
+    xh[::32] *= np.float32(2.0 ** 18)        # one outlier per block: every block of every chunk is flagged
+    w2, x2 = _wx(5, 4096, 64), rng.standard_normal(4096).astype(np.float32)
+    got, got2, goth = _run_group(dev, [{"vx": wq, "y": x}, {"vx": w2, "y": x2}, {"vx": wq, "y": xh}])
+    _check(got, oracle.mul_mat_q4_0_f32(wq, x), (k, n))
+    _check(got2, oracle.mul_mat_q4_0_f32(w2, x2), "short")
+    _check(goth, oracle.mul_mat_q4_0_f32(wq, xh), "outliers")
+    wb, xb, yb = dev.upload(wq), dev.upload(x), dev.alloc(n * 4)
+    dev.dequantize_mul_mat_vec_q4_0(wb, xb, yb, k, n)
+    single = dev.download(yb, np.float32, n)
+    for b in (wb, xb, yb):
+        dev.free(b)
+    assert np.array_equal(got, single)
+
+
 def test_group_shared_activations_and_ragged_row_counts(dev):
     rng = np.random.default_rng(12)
     x = rng.standard_normal(4096).astype(np.float32)
