@@ -39,7 +39,7 @@ ROTATE_BYTES = 1200 << 20
 # HBM bytes per grouped launch (the four products) measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE on
 # this workload, each scaled by what the same counter reads for a device-to-device copy of known size
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); see profiles/gemv_q4_0_group__llama7b_gemv_set.md
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 135045120
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 135240090
 
 
 def q4_bytes(k, n):
