@@ -194,7 +194,9 @@ def test_group_of_six_with_norm_pairs_and_residuals(dev):
         _check(got, _ref_item(it), i)
 
 
-@pytest.mark.parametrize("k,n1,n2", [(4096, 4096, 11008), (256, 100, 33), (11008, 4096, 300), (64, 17, 5)])
+@pytest.mark.parametrize("k,n1,n2", [(4096, 4096, 11008), (256, 100, 33), (11008, 4096, 300), (64, 17, 5),
+                                     # long vectors with many rows (worked in chunks): the producer, then the consumers
+                                     (4160, 4224, 300), (4096, 4160, 4200), (11008, 8192, 2100)])
 def test_group_norm_split_over_two_launches(dev, k, n1, n2):
     """A launch that produces a vector also writes it times the next norm's weight and its sums of squares per 16
     rows; the next launch consumes those instead of normalising: same result as normalising in the second launch."""
