@@ -880,7 +880,7 @@ int32_t prepare_group(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, in
         rows += (int64_t)s.nrows * (s.vx_up ? 2 : 1);
     }
     // Workgroup shape by rows per CU, as for the one-product kernel: few rows -> 16 waves x 1 slot so every SIMD has
-    // work; more rows -> 8 waves x 2 slots, three workgroups resident per CU.  A gate / up pair needs 2 slots per lane.
+    // work; more rows -> 8 waves x 2 slots, four workgroups resident per CU.  A gate / up pair needs 2 slots per lane.
     // One 16-slot row group per workgroup: measured, working through two or four groups per workgroup (which would
     // amortise the activation preparation) loses more to the coarser split of the launch than it saves at every
     // LLaMA-7B shape.
