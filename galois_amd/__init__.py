@@ -65,7 +65,7 @@ class Device:
         self._ctx = ctx
         self._bufs = []
         n = C.c_int32()
-        self._check(self._lib.galois_hip_init_functions(self._ctx, 1, C.byref(n)))
+        self._check(self._lib.galois_hip_init_functions(self._ctx, _abi.ABI_VERSION, C.byref(n)))
         self.n_kernels = n.value
 
     # -- plumbing ---------------------------------------------------------------
@@ -81,6 +81,11 @@ class Device:
             self._bufs = []
             self._lib.galois_hip_destroy(self._ctx)
             self._ctx = None
+
+    OPT_GEMV_F32_ARITHMETIC, OPT_WAIT_SPIN_LIMIT, OPT_WAIT_TARGET_BIAS = 1, 2, 3
+
+    def set_option(self, option, value):
+        self._check(self._lib.galois_hip_set_option(self._ctx, option, value))
 
     def info(self):
         name, arch = C.create_string_buffer(256), C.create_string_buffer(256)

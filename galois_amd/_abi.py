@@ -23,6 +23,8 @@ class GemvItem(C.Structure):
 
 # name -> (restype, argtypes); must list every function the header declares
 PROTOTYPES = {
+    "galois_hip_abi_version": (i32, []),
+    "galois_hip_set_option": (i32, [c_ctx, i32, i32]),
     "galois_hip_create": (i32, [i32, C.POINTER(c_ctx)]),
     "galois_hip_destroy": (i32, [c_ctx]),
     "galois_hip_init_functions": (i32, [c_ctx, i32, C.POINTER(i32)]),
@@ -71,6 +73,8 @@ PROTOTYPES = {
     "galois_hip_mul_mat_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32, i32, i32, C.c_int64, C.c_int64, C.c_int64]),
 }
 
+ABI_VERSION = 2   # GALOIS_HIP_ABI_VERSION this table was written against
+
 _lib = None
 
 
@@ -86,5 +90,8 @@ def load():
         for name, (res, args) in PROTOTYPES.items():
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = res, args
+        if lib.galois_hip_abi_version() != ABI_VERSION:
+            raise ImportError("galois_amd: %s has ABI version %d, these bindings are written against %d -- rebuild it"
+                              % (LIB_PATH, lib.galois_hip_abi_version(), ABI_VERSION))
         _lib = lib
     return _lib

@@ -158,10 +158,10 @@ __device__ __forceinline__ float4 at_store4(_Float16 *p, float4 v) {
 }
 
 // Bounded wait for a counter that other workgroups of the same launch advance (device-coherent reads).  The bound is
-// never reached when the producers are dispatched ahead of the waiters; if it is, the caller poisons its result.
-constexpr int AT_SPIN_LIMIT = 1 << 20;
-__device__ __forceinline__ bool at_wait_ge(const unsigned *p, unsigned target) {
-    for (int it = 0; it < AT_SPIN_LIMIT; it++) {
+// never reached when the producers are dispatched ahead of the waiters; if it is, the caller poisons its result and
+// raises the context's status word.
+__device__ __forceinline__ bool at_wait_ge(const unsigned *p, unsigned target, int spin_limit) {
+    for (int it = 0; it < spin_limit; it++) {
         if ((int)(__hip_atomic_load(const_cast<unsigned *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) >= 0) {
             asm volatile("" ::: "memory");  // what the producers wrote is read after this point
             return true;
@@ -183,14 +183,17 @@ __device__ __forceinline__ float4 at_load4_coherent(const float *p) {
 // ready[H + h], ready[2 H + h] count the workgroups that have stored their rows of head h's q, k, v, and reach
 // `target` when the head's rows are complete.  The cache rows are requested first, then the workgroup waits for q
 // (and, if it holds position n_past, for k and v), which it reads with device-coherent loads.  The workgroup that
-// merges a head returns the three counters to zero.
+// merges a head returns the three counters to zero.  A wait that runs out (spin_limit polls) is agreed on by the whole
+// workgroup: the head's record -- and with it the head's output, whichever workgroup merges it -- becomes NaN in
+// every element, and *status (pinned host memory the context reads after its next wait for the stream) is set.
 template <int LPR, typename CT, int AT_THREADS, bool FUSED>
 __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, const float *__restrict__ k,
                                                const float *__restrict__ v, CT *__restrict__ kc, CT *__restrict__ vc,
                                                float *__restrict__ part, unsigned *__restrict__ done,
                                                float *__restrict__ out, int H, int L, const int32_t *__restrict__ pos,
                                                float freq_scale, float theta_scale, float scale, int h, int s, int S,
-                                               unsigned *ready, unsigned target, int64_t key_stride, int64_t head_stride) {
+                                               unsigned *ready, unsigned target, int64_t key_stride, int64_t head_stride,
+                                               int spin_limit = 0, unsigned *status = nullptr) {
     constexpr int D = LPR * 4, RPL = 64 / LPR, WAVES = AT_THREADS / 64;
     constexpr int KEYS = AT_KEYS;
     constexpr int KPW = KEYS / WAVES;     // keys per wave
@@ -202,6 +205,7 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
     __shared__ float cw[AT_MAX_SPLITS];
     __shared__ float cred[2][WAVES];
     __shared__ unsigned last_flag;
+    __shared__ unsigned gave_up[WAVES];  // FUSED: per wave, whether any of its lanes gave up a wait
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane / LPR, kl = lane % LPR;
     const int l0 = s * KEYS, l1 = min(L, l0 + KEYS), nl = l1 - l0;
@@ -245,16 +249,23 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
     }
     bool arrived = true;
     if (FUSED) {
-        arrived = (int)(seen_q - target) >= 0 || at_wait_ge(ready + h, target);
+        arrived = (int)(seen_q - target) >= 0 || at_wait_ge(ready + h, target, spin_limit);
         asm volatile("" ::: "memory");
         qraw = at_load4_coherent(q + hoff);
         knew_raw = vnew = make_float4(0.f, 0.f, 0.f, 0.f);
         if (l1 - 1 == lnew) {  // the workgroup that holds the new position
-            arrived &= (int)(seen_k - target) >= 0 || at_wait_ge(ready + H + h, target);
-            arrived &= (int)(seen_v - target) >= 0 || at_wait_ge(ready + 2 * H + h, target);
+            arrived &= (int)(seen_k - target) >= 0 || at_wait_ge(ready + H + h, target, spin_limit);
+            arrived &= (int)(seen_v - target) >= 0 || at_wait_ge(ready + 2 * H + h, target, spin_limit);
             asm volatile("" ::: "memory");
             knew_raw = at_load4_coherent(k + hoff);
             vnew = at_load4_coherent(v + hoff);
+        }
+    }
+    if (FUSED) {  // published by the barrier behind the scores; read where the record is written
+        const bool wave_gave_up = __builtin_amdgcn_ballot_w64(!arrived) != 0;
+        if (lane == 0) {
+            gave_up[wave] = wave_gave_up;
+            if (wave_gave_up) __hip_atomic_fetch_or(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
     }
     const float4 qv = rot.apply(qraw);
@@ -335,7 +346,12 @@ __device__ __forceinline__ void attn_decode_wg(const float *__restrict__ q, cons
             o.x += t.x, o.y += t.y, o.z += t.z, o.w += t.w;
         }
         float tot = sred[0];
-        if (FUSED && !arrived) tot = __builtin_nanf("");  // a producer never arrived: the head's output is poisoned
+        if (FUSED) {  // a producer never arrived for some lane of the workgroup: the head's output is poisoned
+            unsigned any = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; w++) any |= gave_up[w];
+            if (any) tot = __builtin_nanf("");
+        }
         if (S == 1) {  // a single split is the whole softmax
             const float inv = 1.0f / tot;
             *reinterpret_cast<float4 *>(out + (size_t)h * D + lane * 4) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);

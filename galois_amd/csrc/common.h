@@ -20,6 +20,12 @@ struct galois_hip_ctx {
     unsigned *attn_done;  // 4 x GH_ATTN_HEADS counters, zero between calls: splits finished per head (decode attention), then
                           // per head the workgroups that have stored its q, its k, its v (the launch that carries both)
     void *attn_static;    // this device's copy of the decode attention's static scratch (attn_decode.hip), found at creation
+                          // (null if the lookup failed: only the entry point that needs it then refuses)
+    unsigned *dev_status;      // one word of pinned host memory that kernels set when a bounded wait inside a launch runs
+    unsigned *dev_status_dev;  // out (the device's address of the same word); read and cleared after every stream wait
+    int32_t wait_spin_limit;   // polls a bounded in-launch wait makes before it gives up (GALOIS_HIP_OPT_WAIT_SPIN_LIMIT)
+    int32_t wait_target_bias;  // added to the count such a wait waits for: test hook (GALOIS_HIP_OPT_WAIT_TARGET_BIAS)
+    bool gemv_f32;             // GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC: one-product GEMV in the reference's f32 arithmetic
     bool capturing;   // between graph_begin_capture and graph_end_capture: nothing may allocate or block
     char last_error[256];
 };
@@ -27,6 +33,7 @@ struct galois_hip_ctx {
 // galois_hip_ctx::scratch holds GH_PARTIAL_FLOATS floats of partial sums.
 constexpr int64_t GH_PARTIAL_FLOATS = 1 << 20;
 constexpr int64_t GH_ATTN_HEADS = 65536;
+constexpr int32_t GH_WAIT_SPIN_DEFAULT = 1 << 20;  // polls of a bounded in-launch wait (a poll and its sleep take about a microsecond)
 
 struct galois_hip_event {
     hipEvent_t ev;
@@ -76,6 +83,9 @@ static inline int32_t gh_hip(galois_hip_ctx *ctx, hipError_t e, const char *what
     } while (0)
 
 #define GH_LAUNCH_CHECK(ctx, what) return gh_hip((ctx), hipGetLastError(), (what))
+
+// device.hip: after a wait for the stream, reports (and clears) what kernels left in the context's status word.
+int32_t gh_check_device_status(galois_hip_ctx *ctx);
 
 // attn_decode.hip: looks up the device's copy of the attention's static scratch (the context's device is current).
 int32_t gh_attn_static_init(galois_hip_ctx *ctx);

@@ -3,6 +3,21 @@
 #include "common.h"
 
 
+// Called once the stream has drained.  A kernel whose bounded wait for other workgroups of its launch ran out has
+// set the context's status word (and poisoned its own result with NaN); the workgroups it gave up on may have counted
+// themselves after the counters were returned to zero, so the counters are cleared here before anything else runs.
+int32_t gh_check_device_status(galois_hip_ctx *ctx) {
+    if (!ctx->dev_status || __atomic_load_n(ctx->dev_status, __ATOMIC_ACQUIRE) == 0) return GALOIS_HIP_OK;
+    __atomic_store_n(ctx->dev_status, 0u, __ATOMIC_RELEASE);
+    hipError_t e = hipMemsetAsync(ctx->attn_done, 0, 4 * GH_ATTN_HEADS * sizeof(unsigned), ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return gh_hip(ctx, e, "clearing the wait counters");
+    return gh_fail(ctx, GALOIS_HIP_E_DEVICE_WAIT,
+                   "qkv_attn_decode: a workgroup gave up waiting for the products of its launch; the attention output of "
+                   "that call is NaN and what was launched after it on this context is not to be trusted (the counters "
+                   "have been cleared: the context can be used again)");
+}
+
 extern "C" {
 
 const char *galois_hip_status_string(int32_t s) {
@@ -14,6 +29,7 @@ const char *galois_hip_status_string(int32_t s) {
         case GALOIS_HIP_E_ORDINAL: return "no such device";
         case GALOIS_HIP_E_UNSUPPORTED: return "unsupported combination";
         case GALOIS_HIP_E_ARCH: return "device is not gfx950";
+        case GALOIS_HIP_E_DEVICE_WAIT: return "a bounded wait inside a launch ran out";
         default: return s > 0 ? hipGetErrorString((hipError_t)s) : "unknown status";
     }
 }
@@ -41,6 +57,11 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     ctx->attn_done = nullptr;
     ctx->attn_static = nullptr;
     ctx->capturing = false;
+    ctx->dev_status = nullptr;
+    ctx->dev_status_dev = nullptr;
+    ctx->wait_spin_limit = GH_WAIT_SPIN_DEFAULT;
+    ctx->wait_target_bias = 0;
+    ctx->gemv_f32 = false;
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         delete ctx;
@@ -51,11 +72,19 @@ int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out) {
     if (e == hipSuccess) e = hipMemsetAsync(ctx->scratch, 0, scratch_bytes, ctx->stream);
     if (e == hipSuccess) e = hipMalloc((void **)&ctx->attn_done, 4 * GH_ATTN_HEADS * sizeof(unsigned));
     if (e == hipSuccess) e = hipMemsetAsync(ctx->attn_done, 0, 4 * GH_ATTN_HEADS * sizeof(unsigned), ctx->stream);
+    // the status word lives in pinned host memory that the device writes directly: reading it costs the host nothing
+    if (e == hipSuccess) e = hipHostMalloc((void **)&ctx->dev_status, 64, hipHostMallocMapped);
+    if (e == hipSuccess) {
+        *ctx->dev_status = 0;
+        e = hipHostGetDevicePointer((void **)&ctx->dev_status_dev, ctx->dev_status, 0);
+    }
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-    if (e == hipSuccess && gh_attn_static_init(ctx) != GALOIS_HIP_OK) e = hipErrorNotFound;
+    // only galois_hip_attn_decode_f32_static needs the static scratch; without it that entry point refuses by itself
+    if (e == hipSuccess) (void)gh_attn_static_init(ctx);
     if (e != hipSuccess) {
         if (ctx->scratch) (void)hipFree(ctx->scratch);
         if (ctx->attn_done) (void)hipFree(ctx->attn_done);
+        if (ctx->dev_status) (void)hipHostFree(ctx->dev_status);
         (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return (int32_t)e;
@@ -72,9 +101,31 @@ int32_t galois_hip_destroy(galois_hip_ctx *ctx) {
     for (void *p : ctx->ws_retired) (void)hipFree(p);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->attn_done) (void)hipFree(ctx->attn_done);
+    if (ctx->dev_status) (void)hipHostFree(ctx->dev_status);
     hipError_t e = hipStreamDestroy(ctx->stream);
     delete ctx;
     return (int32_t)e;
+}
+
+int32_t galois_hip_abi_version(void) { return GALOIS_HIP_ABI_VERSION; }
+
+int32_t galois_hip_set_option(galois_hip_ctx *ctx, int32_t option, int32_t value) {
+    GH_REQUIRE_CTX(ctx);
+    switch (option) {
+        case GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC:
+            ctx->gemv_f32 = value != 0;
+            return GALOIS_HIP_OK;
+        case GALOIS_HIP_OPT_WAIT_SPIN_LIMIT:
+            GH_REQUIRE(ctx, value >= 0, GALOIS_HIP_E_SHAPE, "set_option: the poll limit is 0 (the default) or positive");
+            ctx->wait_spin_limit = value > 0 ? value : GH_WAIT_SPIN_DEFAULT;
+            return GALOIS_HIP_OK;
+        case GALOIS_HIP_OPT_WAIT_TARGET_BIAS:
+            GH_REQUIRE(ctx, value >= 0 && value <= 1, GALOIS_HIP_E_SHAPE, "set_option: the target bias is 0 or 1");
+            ctx->wait_target_bias = value;
+            return GALOIS_HIP_OK;
+        default:
+            return gh_fail(ctx, GALOIS_HIP_E_UNSUPPORTED, "set_option: unknown option");
+    }
 }
 
 int32_t galois_hip_init_functions(galois_hip_ctx *ctx, int32_t abi_version, int32_t *n_kernels) {
@@ -149,7 +200,9 @@ int32_t galois_hip_dtoh_sync_copy(galois_hip_ctx *ctx, void *dst_host, const voi
     GH_BIND(ctx);
     hipError_t e = hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream);
     if (e != hipSuccess) return gh_hip(ctx, e, "hipMemcpyAsync(D2H)");
-    return gh_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipStreamSynchronize");
+    return gh_check_device_status(ctx);
 }
 
 int32_t galois_hip_dtod_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
@@ -178,7 +231,9 @@ int32_t galois_hip_synchronize(galois_hip_ctx *ctx) {
     GH_REQUIRE_CTX(ctx);
     GH_NOT_CAPTURING(ctx, "synchronize");
     GH_BIND(ctx);
-    return gh_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    const hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipStreamSynchronize");
+    return gh_check_device_status(ctx);
 }
 
 int32_t galois_hip_event_create(galois_hip_ctx *ctx, galois_hip_event **out) {

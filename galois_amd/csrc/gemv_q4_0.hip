@@ -934,6 +934,8 @@ struct fa_args {
     const int32_t *pos;
     int32_t H, L, S, gemv_blocks;
     uint32_t target;
+    int32_t spin_limit;  // polls of a bounded wait
+    unsigned *status;    // the context's status word (pinned host memory): set when a wait runs out
     float freq_scale, theta_scale, scale;
     int64_t key_stride, head_stride;  // of the caches, in elements
 };
@@ -957,7 +959,7 @@ __global__ __launch_bounds__(FA_WAVES * 64, 4) void qkv_attn_decode_fused(const 
         attn_decode_wg<FA_HEAD_DIM / 4, CT, FA_WAVES * 64, true>(a.dst[0], a.dst[1], a.dst[2], b.kc, b.vc, b.part, b.done, b.out,
                                                                  b.H, b.L, b.pos, b.freq_scale, b.theta_scale, b.scale,
                                                                  t % b.H, t / b.H, b.S, b.ready, b.target, b.key_stride,
-                                                                 b.head_stride);
+                                                                 b.head_stride, b.spin_limit, b.status);
     }
 }
 
@@ -999,7 +1001,9 @@ int32_t launch_qkv_attn(galois_hip_ctx *ctx, const galois_hip_gemv_item *items, 
     b.kc = k_cache, b.vc = v_cache, b.part = (float *)ctx->scratch, b.out = out;
     b.done = ctx->attn_done, b.ready = ctx->attn_done + GH_ATTN_HEADS, b.pos = pos;
     b.H = n_head, b.L = L, b.S = S, b.gemv_blocks = (int32_t)plan.blocks;
-    b.target = FA_HEAD_DIM / (FA_WAVES * FA_R);  // product workgroups per head
+    b.target = FA_HEAD_DIM / (FA_WAVES * FA_R) + (uint32_t)ctx->wait_target_bias;  // product workgroups per head
+    b.spin_limit = ctx->wait_spin_limit, b.status = ctx->dev_status_dev;
+    GH_REQUIRE(ctx, b.status != nullptr, GALOIS_HIP_E_UNSUPPORTED, "qkv_attn_decode: the context has no status word");
     b.freq_scale = freq_scale, b.theta_scale = theta_scale, b.scale = scale;
     b.key_stride = head_major_n_ctx ? head_dim : (int64_t)n_head * head_dim;
     b.head_stride = head_major_n_ctx ? (int64_t)head_major_n_ctx * head_dim : head_dim;
@@ -1035,7 +1039,8 @@ extern "C" int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, c
     GH_REQUIRE(ctx, gh_aligned(vx, 2) && gh_aligned(y, 4) && gh_aligned(dst, 4), GALOIS_HIP_E_ALIGN,
                "dequantize_mul_mat_vec_q4_0");
     GH_BIND(ctx);
-    const bool fast = (ncols % 64 == 0) && gh_aligned(vx, 4) && gh_aligned(y, 8);
+    // GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC: the caller asked for the reference's f32 multiply-add, weight by weight
+    const bool fast = (ncols % 64 == 0) && gh_aligned(vx, 4) && gh_aligned(y, 8) && !ctx->gemv_f32;
     if (fast) {
         const int nslots = ncols / 64;
         // Workgroup shape by rows per CU: few rows -> 16 waves x 1 row so every SIMD has work and the

@@ -42,6 +42,10 @@ GResult CudaDevice::create(int ordinal, std::shared_ptr<CudaDevice> *out) {
     int32_t st = galois_hip_create(ordinal, &ctx);
     if (st != 0) return err(GError::DeviceError, std::string("CudaDevice::new: ") + galois_hip_status_string(st));
     int32_t n = 0;
+    if (galois_hip_abi_version() != GALOIS_HIP_ABI_VERSION) {
+        galois_hip_destroy(ctx);
+        return err(GError::DeviceError, "libgalois_hip: ABI version differs from the header this mirror was built against");
+    }
     st = galois_hip_init_functions(ctx, GALOIS_HIP_ABI_VERSION, &n);
     if (st != 0) {
         galois_hip_destroy(ctx);
@@ -189,11 +193,14 @@ static GResult matmul_f32(const CudaDevice &dev, const Tensor &a, const Tensor &
         return err(GError::Unimplemented, "matmul f32: src1 and dst must be contiguous");
     // an F16 src0 is the (F16, F32) -> F32 arm that the reference hands to cuBLAS (CudaMatMul::f_x_y_y,
     // src/cuda.rs:881-992): the same views, the a operand widened exactly
-    auto fn = a.dtype() == GGmlType::F16 ? (decltype(&galois_hip_mul_mat_f16_f32))galois_hip_mul_mat_f16_f32
-                                         : (decltype(&galois_hip_mul_mat_f16_f32))galois_hip_mul_mat_f32;
-    return dev.check(fn(dev.ctx(), a.data(), (const float *)b.data(), (float *)dst.data(), (int32_t)ad.shape[0],
-                        (int32_t)ad.shape[1], (int32_t)bd.shape[1], (int32_t)ad.shape[2], (int32_t)bd.shape[2],
-                        (int64_t)ad.stride[0], (int64_t)ad.stride[1], (int64_t)ad.stride[2]));
+    const int32_t K = (int32_t)ad.shape[0], N = (int32_t)ad.shape[1], M = (int32_t)bd.shape[1];
+    const int32_t ne02 = (int32_t)ad.shape[2], ne12 = (int32_t)bd.shape[2];
+    const int64_t s0 = (int64_t)ad.stride[0], s1 = (int64_t)ad.stride[1], s2 = (int64_t)ad.stride[2];
+    if (a.dtype() == GGmlType::F16)
+        return dev.check(galois_hip_mul_mat_f16_f32(dev.ctx(), a.data(), (const float *)b.data(), (float *)dst.data(), K, N, M,
+                                                    ne02, ne12, s0, s1, s2));
+    return dev.check(galois_hip_mul_mat_f32(dev.ctx(), (const float *)a.data(), (const float *)b.data(), (float *)dst.data(),
+                                            K, N, M, ne02, ne12, s0, s1, s2));
 }
 
 // galois_matmul, src/op.rs:3093-3111 -> CudaMatMul.map -> f_q_f32_f32 (src/cuda.rs:994-1139).

@@ -33,7 +33,10 @@
 extern "C" {
 #endif
 
-#define GALOIS_HIP_ABI_VERSION 1
+/* Changes whenever the argument list of an exported function changes (2: n_table_rows of get_rows_q4_0,
+ * head_major_n_ctx of the attention calls, galois_hip_abi_version / galois_hip_set_option added).  A binding compares
+ * the value it was written against with galois_hip_abi_version() before its first call. */
+#define GALOIS_HIP_ABI_VERSION 2
 
 #define GALOIS_HIP_OK 0
 #define GALOIS_HIP_E_NULL (-1)      /* a required pointer is NULL */
@@ -42,12 +45,20 @@ extern "C" {
 #define GALOIS_HIP_E_ORDINAL (-4)   /* no such device */
 #define GALOIS_HIP_E_UNSUPPORTED (-5) /* the reference leaves this combination todo!() and so do we */
 #define GALOIS_HIP_E_ARCH (-6)      /* the device is not gfx950 */
+#define GALOIS_HIP_E_DEVICE_WAIT (-7) /* reported by synchronize / *_sync_copy: a workgroup of galois_hip_qkv_attn_decode_*
+                                       * gave up a bounded wait for other workgroups of its launch.  The attention output of
+                                       * that call is NaN, later launches on the context may have read stale vectors; the
+                                       * status is reported once, the context is usable again afterwards */
 
 typedef struct galois_hip_ctx galois_hip_ctx;
 typedef struct galois_hip_event galois_hip_event;
 typedef struct galois_hip_graph galois_hip_graph;
 
 /* ---- device / stream / buffer layer -------------------------------------- */
+
+/* GALOIS_HIP_ABI_VERSION of the library that was loaded (valid without a context; no counterpart in the reference,
+ * whose kernels are looked up by name at run time, src/cuda.rs:304-307). */
+int32_t galois_hip_abi_version(void);
 
 /* CudaDevice::new(ordinal), src/cuda.rs:221-229: bind a device, create its stream. */
 int32_t galois_hip_create(int32_t ordinal, galois_hip_ctx **out);
@@ -56,6 +67,18 @@ int32_t galois_hip_destroy(galois_hip_ctx *ctx);
  * the library, so nothing is loaded; this checks the ABI version and that the
  * device can run them, and returns the number of kernels in *n_kernels. */
 int32_t galois_hip_init_functions(galois_hip_ctx *ctx, int32_t abi_version, int32_t *n_kernels);
+/* Per-context switches (no counterpart in the reference).  Unknown options return GALOIS_HIP_E_UNSUPPORTED.
+ *   GEMV_F32_ARITHMETIC (0 / 1, default 0): galois_hip_dequantize_mul_mat_vec_q4_0 multiplies and adds in f32, weight by
+ *     weight, as dequantize_mul_mat_vec_q4_0 does (matmul.cu:72-100), instead of the block-scaled fixed-point dot
+ *     (same results within the 1e-4 bar; several times slower).  The grouped and fused launches are not affected.
+ *   WAIT_SPIN_LIMIT (polls; 0 restores the default of 2^20, about a second) and WAIT_TARGET_BIAS (0 / 1): the bound
+ *     of the waits inside galois_hip_qkv_attn_decode_* and an offset added to the count they wait for.  For tests of
+ *     the give-up path only: with bias 1 every wait runs out, every kernel still ends normally, the call's output is
+ *     NaN and the next synchronize returns GALOIS_HIP_E_DEVICE_WAIT. */
+#define GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC 1
+#define GALOIS_HIP_OPT_WAIT_SPIN_LIMIT 2
+#define GALOIS_HIP_OPT_WAIT_TARGET_BIAS 3
+int32_t galois_hip_set_option(galois_hip_ctx *ctx, int32_t option, int32_t value);
 /* Text of the last non-zero status on this context ("" if none); never NULL. */
 const char *galois_hip_last_error(const galois_hip_ctx *ctx);
 /* Name for a status code of this ABI (valid without a context). */
@@ -77,7 +100,8 @@ int32_t galois_hip_dtoh_sync_copy(galois_hip_ctx *ctx, void *dst_host, const voi
 int32_t galois_hip_dtod_copy(galois_hip_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
 int32_t galois_hip_dtod_copy_2d(galois_hip_ctx *ctx, void *dst_dev, size_t dpitch, const void *src_dev,
                                 size_t spitch, size_t width_bytes, size_t height);
-/* Stream synchronisation (implicit in the reference's to_cpu_tensor, src/lib.rs:2314). */
+/* Stream synchronisation (implicit in the reference's to_cpu_tensor, src/lib.rs:2314).  This call and the two
+ * *_sync_copy calls also report GALOIS_HIP_E_DEVICE_WAIT (above) for work that has finished. */
 int32_t galois_hip_synchronize(galois_hip_ctx *ctx);
 
 /* Timing on the context's stream (the reference has none: dead SystemTime pairs, src/op.rs:1392-1395). */
@@ -114,7 +138,13 @@ int32_t galois_hip_dequantize_row_q4_0(galois_hip_ctx *ctx, const void *x, float
  * (src/cuda.rs:1011-1034 -> galois-kernels/src/matmul.cu:45-117), same argument
  * order: dst[row] = sum_col (q-8)*d * y[col], f32.  vx: nrows rows of ncols/32
  * Q4_0 blocks; ncols % 32 == 0; vx 2-byte aligned, y/dst 4-byte aligned.
- * The caller loops ne12*ne13 batch slices exactly as src/cuda.rs:1026-1034. */
+ * The caller loops ne12*ne13 batch slices exactly as src/cuda.rs:1026-1034.
+ * Arithmetic: when ncols % 64 == 0 and vx is 4-byte, y 8-byte aligned, the activations are rounded per block of 32 to
+ * 18 bits below the block's largest one (blocks that this would leave too coarse carry a second, finer grid) and the
+ * products are exact integer dots scaled in f32: within 1e-4 of the f64 dequantize-then-dot result (max error over
+ * max |result|, and relative L2) for every input tested, with ONE stated exception -- a vector whose every block has its
+ * largest activation below 2^-108 keeps 13 bits per block and stays within 5e-4.  Otherwise, and always when
+ * GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC is set, plain f32 multiply-add as in the reference kernel. */
 int32_t galois_hip_dequantize_mul_mat_vec_q4_0(galois_hip_ctx *ctx, const void *vx, const float *y,
                                                float *dst, int32_t ncols, int32_t nrows);
 
@@ -279,7 +309,8 @@ int32_t galois_hip_attn_decode_f16kv(galois_hip_ctx *ctx, const float *q, const 
  * q, k and v vectors of n_head * head_dim floats (written as by the group call, and read by the attention part).
  * The attention's workgroups follow the products' in the grid, request their cache rows while the last products
  * still stream, and wait -- bounded -- only for their own head's rows of q (k and v where position n_past lives);
- * should a wait ever run out, that head's output is NaN.  q, k, v and the appended cache rows equal those of the two
+ * should a wait ever run out, that head's whole output is NaN, the context's status word is set and the next synchronize
+ * or *_sync_copy returns GALOIS_HIP_E_DEVICE_WAIT (once) after returning the counters to zero.  q, k, v and the appended cache rows equal those of the two
  * calls issued one after the other bit for bit (when the group call would run few rows in its 16-wave shape: up to the
  * order in which a normalising product adds its squares), the output up to the order of its f32 sums.  head_dim 128; the products are plain or normalising (no vx_up, residual, dst_scaled, sumsq_out); dst
  * 16-byte aligned; ncols <= 11776; otherwise the limits of both calls apply. */

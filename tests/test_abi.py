@@ -118,9 +118,16 @@ def test_rust_binding_block_matches_the_header():
 def test_status_strings_without_device():
     lib = _abi.load()
     assert lib.galois_hip_status_string(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5, -6):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert lib.galois_hip_status_string(code) not in (b"", b"unknown status")
     assert lib.galois_hip_status_string(-99) == b"unknown status"
+
+
+def test_abi_version_is_exported_and_matches_the_header():
+    lib = _abi.load()
+    m = re.search(r"#define GALOIS_HIP_ABI_VERSION (\d+)", open(HEADER).read())
+    assert lib.galois_hip_abi_version() == int(m.group(1)) == _abi.ABI_VERSION
+    assert lib.galois_hip_set_option(None, 1, 1) == -1
 
 
 def test_null_context_is_an_error_not_a_crash():

@@ -66,11 +66,19 @@ def test_gemm_prefill_config(dev):
     m, k, n = 512, 4096, 11008
     wq, x = _case(3, m, k, n)
     got = _gemm(dev, wq, x)
-    # the oracle on a column sample (full 512x11008x4096 in f64 takes too long on the CPU here)
+    # every one of the 512 x 11008 outputs against dequantize-then-GEMM in f64 (numpy's matmul on the independent
+    # vectorised dequantizer of tests/npref.py) ...
+    full = x.astype(np.float64) @ npref.q4_0_dequant(wq).astype(np.float64).T
+    emax, el2 = npref.rel_err(got, full)
+    worst_col = float(np.max(np.max(np.abs(got - full), axis=0)) / np.max(np.abs(full)))
+    print("prefill, all outputs: max_rel=%.3g l2_rel=%.3g (worst column %.3g)" % (emax, el2, worst_col))
+    assert emax < TOL and el2 < TOL
+    # ... and the C oracle on a column sample, which ties the numpy reference to the oracle at this size
     cols = np.random.default_rng(4).choice(n, 512, replace=False)
     ref = oracle.mul_mat_q4_0_f32(wq[cols], x)
+    emax, el2 = npref.rel_err(full[:, cols], ref)
+    assert emax < 1e-6 and el2 < 1e-6
     emax, el2 = npref.rel_err(got[:, cols], ref)
-    print("prefill max_rel=%.3g l2_rel=%.3g" % (emax, el2))
     assert emax < TOL and el2 < TOL
     # size-independent property at the full size: linearity in X (exact except where halving
     # pushes an fp16 activation into the subnormal range)

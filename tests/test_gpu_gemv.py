@@ -196,6 +196,31 @@ def test_gemv_subnormal_blocks_next_to_large_ones(dev):
     assert emax < 5e-4 and el2 < 5e-4
 
 
+def test_gemv_in_reference_f32_arithmetic_on_request(dev):
+    """GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC: the one-product call multiplies and adds in f32, weight by weight, as the
+    reference kernel does (matmul.cu:72-100), on the shapes the fixed-point kernel would otherwise take.  Both meet
+    the 1e-4 bar; the vector that lies entirely below 2^-108 -- the fixed-point kernel's one stated exception --
+    is inside it in f32 arithmetic."""
+    for k, n in ((4096, 4096), (11008, 257)):
+        wq, x = _case(k + n, k, n)
+        ref = oracle.mul_mat_q4_0_f32(wq, x)
+        fixed = _gemv(dev, wq, x)
+        dev.set_option(dev.OPT_GEMV_F32_ARITHMETIC, 1)
+        try:
+            f32 = _gemv(dev, wq, x)
+            tiny = (x * np.float32(2.0 ** -112)).astype(np.float32)
+            f32_tiny = _gemv(dev, wq, tiny)
+        finally:
+            dev.set_option(dev.OPT_GEMV_F32_ARITHMETIC, 0)
+        for got in (fixed, f32):
+            emax, el2 = npref.rel_err(got, ref)
+            assert emax < TOL and el2 < TOL, (k, n, emax, el2)
+        assert not np.array_equal(fixed, f32), "the option selected the same kernel"
+        emax, el2 = npref.rel_err(f32_tiny, oracle.mul_mat_q4_0_f32(wq, tiny))
+        assert emax < TOL and el2 < TOL, ("2^-112", emax, el2)
+        assert np.array_equal(_gemv(dev, wq, x), fixed), "the option is off again"
+
+
 def test_gemv_argument_errors(dev):
     from galois_amd import GaloisHipError
     buf = dev.alloc(4096)

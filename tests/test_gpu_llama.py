@@ -262,3 +262,85 @@ def test_full_width_layers_at_kv_length_2048(gdev):
         dec.decode(31999, 2047, fused)
         _check(dec.logits(), ref, 1e-4)
     dec.close()
+
+
+def _normal_f32(seed, count, scale, threads=8):
+    """count f32 draws of N(0, scale^2) from `threads` independent streams filled in parallel."""
+    from concurrent.futures import ThreadPoolExecutor
+    out = np.empty(count, np.float32)
+    bounds = np.linspace(0, count, threads + 1).astype(np.int64)
+
+    def fill(t):
+        g = np.random.default_rng([seed, t])
+        g.standard_normal(out=out[bounds[t]:bounds[t + 1]], dtype=np.float32)
+        out[bounds[t]:bounds[t + 1]] *= np.float32(scale)
+
+    with ThreadPoolExecutor(threads) as ex:
+        list(ex.map(fill, range(threads)))
+    return out
+
+
+def test_32_layers_at_kv_length_2048_against_the_oracle(gdev):
+    """BASELINE configs[4] at its stated depth: 32 layers of distinct N(0, 0.02) weights quantized to Q4_0 (by the
+    oracle, on the host), d_model 4096, 32 heads, FFN 11008, vocab 32000, one token attending over 2048 cached
+    positions, against the oracle's op-by-op step in f64 dot products.  What accumulates over 225 products of the
+    block-fixed-point matvec is measured here against arithmetic that does not share it.  Every layer's cache starts
+    from the same 2047 rows (the step appends its own row 2047 to each before reading it), which keeps the host side
+    at two 32 MB arrays; the weights differ from layer to layer."""
+    from concurrent.futures import ThreadPoolExecutor
+    hp = dict(n_vocab=32000, n_embd=4096, n_head=32, n_layer=32, n_ff=11008, n_ctx=2048, rms_eps=1e-6, freq_base=10000.0)
+    e, f, v, c = hp["n_embd"], hp["n_ff"], hp["n_vocab"], hp["n_ctx"]
+    shapes = {"wq": (e, e), "wk": (e, e), "wv": (e, e), "wo": (e, e), "w_gate": (f, e), "w_up": (f, e), "w_down": (e, f)}
+    seed = [1000]
+
+    def q(rows, cols):   # rows quantized in parallel slabs (the oracle's quantizer is one thread per call)
+        seed[0] += 1
+        w = _normal_f32(seed[0], rows * cols, 0.02).reshape(rows, cols)
+        slabs = np.array_split(np.arange(rows), 8)
+        with ThreadPoolExecutor(8) as ex:
+            parts = list(ex.map(lambda r: oracle.quantize_q4_0(w[r[0]:r[-1] + 1]), slabs))
+        return np.concatenate(parts)
+
+    rng = np.random.default_rng(77)
+    print("32-layer step: drawing and quantizing weights", flush=True)
+    w = {"tok_embd": q(v, e), "output": q(v, e), "out_norm": (1 + 0.1 * rng.standard_normal(e)).astype(np.float32),
+         "layers": []}
+    for _ in range(hp["n_layer"]):
+        lw = {n: q(*shapes[n]) for n in LAYER_Q}
+        lw["attn_norm"] = (1 + 0.1 * rng.standard_normal(e)).astype(np.float32)
+        lw["ffn_norm"] = (1 + 0.1 * rng.standard_normal(e)).astype(np.float32)
+        w["layers"].append(lw)
+    kc0 = _normal_f32(5, c * e, 1.0).reshape(c, e)
+    vc0 = _normal_f32(6, c * e, 1.0).reshape(c, e)
+    tok, n_past = 31999, c - 1
+    print("32-layer step: oracle", flush=True)
+    kc_ref = [kc0.copy()] * hp["n_layer"]   # one array behind every layer: each layer rewrites row n_past before it reads
+    vc_ref = [vc0.copy()] * hp["n_layer"]
+    ref = _ref_step(w, hp, kc_ref, vc_ref, tok, n_past)
+    assert np.all(np.isfinite(ref))
+    dec = g.LlamaDecoder(gdev, **hp)
+    for n in ("tok_embd", "output", "out_norm"):
+        dec.tensor(n).write(w[n])
+    for i, lw in enumerate(w["layers"]):
+        for n, a in lw.items():
+            dec.tensor(n, i).write(a)
+
+    def load_caches():
+        for i in range(hp["n_layer"]):
+            dec.tensor("k_cache", i).write(kc0)
+            dec.tensor("v_cache", i).write(vc0)
+
+    worst = {}
+    for fused in (0, 4, 5):
+        print("32-layer step: plan %d" % fused, flush=True)
+        load_caches()
+        dec.decode(tok, n_past, fused)
+        worst[fused] = npref.rel_err(dec.logits(), ref)
+    load_caches()
+    dec.capture(tok, n_past, 5)
+    dec.replay()
+    worst["graph5"] = npref.rel_err(dec.logits(), ref)
+    dec.close()
+    print("32-layer logits vs the oracle (max-rel, l2-rel):", worst, flush=True)
+    for plan, (emax, el2) in worst.items():
+        assert emax < 1e-4 and el2 < 1e-4, (plan, emax, el2)

@@ -135,3 +135,57 @@ def test_qkv_attn_repeated_calls(dev):
     _case(dev, 32, 4096, 1500, 2, False, seed=5, repeats=6)
     _case(dev, 5, 256, 700, 1, False, seed=6, repeats=3)
     _case(dev, 32, 4096, 100, 1, True, seed=7, repeats=3)
+
+
+@pytest.mark.parametrize("H,K,n_past", [(32, 4096, 2047), (3, 256, 40)])
+def test_a_wait_that_runs_out_is_reported_and_leaves_the_context_usable(dev, H, K, n_past):
+    """The give-up path of the waits inside the launch, forced from the host: the attention workgroups wait for one
+    count more than the products can reach, with a bound of a few polls, so every wait runs out and every kernel
+    still ends normally.  Every head's output is NaN in all its elements, the products themselves are right, the next
+    synchronize reports GALOIS_HIP_E_DEVICE_WAIT exactly once, and the same call afterwards -- with the default
+    settings -- gives what it gave before, bit for bit (the counters the late products left non-zero are cleared)."""
+    from galois_amd import GaloisHipError
+    D = 128
+    E = H * D
+    rng = np.random.default_rng(90 + H)
+    ws = [dev.upload(oracle.quantize_q4_0((rng.standard_normal((E, K)) * 0.05).astype(np.float32))) for _ in range(3)]
+    x = dev.upload(rng.standard_normal(K).astype(np.float32))
+    kc0 = rng.standard_normal((n_past + 1, E)).astype(np.float32)
+    vc0 = rng.standard_normal((n_past + 1, E)).astype(np.float32)
+    pos = dev.upload(np.array([n_past], np.int32))
+    q, k, v, out = (dev.alloc(E * 4) for _ in range(4))
+    kc, vc = dev.upload(kc0), dev.upload(vc0)
+    items = dev.gemv_items([{"vx": w, "y": x, "dst": d, "ncols": K, "nrows": E} for w, d in zip(ws, (q, k, v))])
+    args = (items, kc, vc, out, H, D, n_past, pos, 1.0, 10000.0 ** (-2.0 / D), D ** -0.5)
+
+    def run():
+        dev.upload(kc0, kc), dev.upload(vc0, vc)
+        dev.qkv_attn_decode(*args)
+        dev.synchronize()
+        return [dev.download(b, np.float32, E) for b in (q, k, v, out)]
+
+    good = run()
+    assert np.all(np.isfinite(good[3]))
+    print("give-up case H=%d K=%d n_past=%d" % (H, K, n_past), flush=True)
+    dev.set_option(dev.OPT_WAIT_SPIN_LIMIT, 4)
+    dev.set_option(dev.OPT_WAIT_TARGET_BIAS, 1)
+    try:
+        dev.upload(kc0, kc), dev.upload(vc0, vc)
+        dev.qkv_attn_decode(*args)
+        with pytest.raises(GaloisHipError) as ei:
+            dev.synchronize()
+        assert ei.value.status == -7
+        dev.synchronize()                                   # reported once
+        bad = [dev.download(b, np.float32, E) for b in (q, k, v, out)]
+        assert np.all(np.isnan(bad[3])), "every element of every head is poisoned"
+        for a, b in zip(good[:3], bad[:3]):                 # the products do not depend on the waits
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    finally:
+        dev.set_option(dev.OPT_WAIT_TARGET_BIAS, 0)
+        dev.set_option(dev.OPT_WAIT_SPIN_LIMIT, 0)
+    for _ in range(2):
+        again = run()
+        for a, b in zip(good, again):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    for b in ws + [x, pos, q, k, v, out, kc, vc]:
+        dev.free(b)
