@@ -57,5 +57,24 @@ def build_host(verbose=False):
     return HOST_LIB
 
 
+SAN_FLAGS = ["-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined"]
+
+
+def build_host_sanitized(verbose=False):
+    """The host mirror under the address and undefined-behaviour sanitizers (host code only, for CPU tests: it parses
+    model files and does pointer arithmetic over tensor views).  Goes to build/san/ and is never loaded by default;
+    GALOIS_HOST_LIB points an interpreter that has the sanitizer runtime preloaded at it."""
+    out_dir = os.path.join(OBJ, "san")
+    os.makedirs(out_dir, exist_ok=True)
+    out = os.path.join(out_dir, "libgalois_host.so")
+    srcs = sorted(glob.glob(os.path.join(HERE, "host", "*.cpp")))
+    cmd = ["g++", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", *SAN_FLAGS, "-o", out, *srcs,
+           "-L" + HERE, "-lgalois_hip", "-Wl,-rpath," + HERE]
+    subprocess.check_call(cmd)
+    if verbose:
+        print("built", out)
+    return out
+
+
 if __name__ == "__main__":
     build(verbose=True, extra=sys.argv[1:])

@@ -33,6 +33,13 @@ void *galois_host_device_new(int ordinal) {
     return d;
 }
 void *galois_host_device_cpu() { return new Device(); }
+// galois_hip_set_option on the device's context (a Cpu device has none)
+int galois_host_device_set_option(void *d, int option, int value) {
+    auto *dev = (Device *)d;
+    if (!dev->is_gpu()) return fail(GError{GError::Unimplemented, "set_option: a Cpu device has no options"});
+    GResult r = dev->gpu->check(galois_hip_set_option(dev->gpu->ctx(), option, value));
+    return r.ok() ? 0 : fail(r);
+}
 void galois_host_device_free(void *d) { delete (Device *)d; }
 
 void *galois_host_tensor_from_raw(void *dev, const void *bytes, size_t nbytes, size_t n_dims, const size_t *shape, int dtype) {

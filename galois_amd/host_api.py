@@ -10,7 +10,9 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libgalois_host.so")
+# GALOIS_HOST_LIB: another build of the same library (the address / undefined-behaviour sanitizer build that
+# tests/test_sanitizers.py makes with galois_amd.build.build_host_sanitized)
+LIB_PATH = os.environ.get("GALOIS_HOST_LIB") or os.path.join(HERE, "libgalois_host.so")
 
 F32, F16, Q4_0, I32 = 0, 1, 2, 18
 _NP = {F32: np.float32, F16: np.float16, Q4_0: np.uint8, I32: np.int32}
@@ -38,6 +40,7 @@ def lib():
         for name, res, args in (
                 ("galois_host_device_new", vp, [C.c_int]), ("galois_host_device_cpu", vp, []),
                 ("galois_host_device_free", None, [vp]),
+                ("galois_host_device_set_option", C.c_int, [vp, C.c_int, C.c_int]),
                 ("galois_host_tensor_from_raw", vp, [vp, vp, sz, sz, C.POINTER(sz), C.c_int]),
                 ("galois_host_tensor_zeros", vp, [vp, sz, C.POINTER(sz), C.c_int]),
                 ("galois_host_tensor_view", vp, [vp, sz, sz, C.POINTER(sz)]),
@@ -110,6 +113,10 @@ class Device:
         if not h:
             _raise(3)
         return Device(h)
+
+    def set_option(self, option, value):
+        """``galois_hip_set_option`` on the device's context (option numbers: include/galois_hip.h)."""
+        _call(lib().galois_host_device_set_option(self.h, option, value))
 
 
 class Tensor:

