@@ -196,6 +196,28 @@ class Device:
     def mul_mat_q4_0_f32(self, W, X, Y, K, N, M):
         self._check(self._lib.galois_hip_mul_mat_q4_0_f32(self._ctx, _ptr(W), _ptr(X), _ptr(Y), K, N, M))
 
+    def f16_panel_bytes(self, K, M):
+        n = C.c_int64()
+        self._check(self._lib.galois_hip_f16_panel_bytes(K, M, C.byref(n)))
+        return n.value
+
+    def f32_to_f16_panel(self, x, panel, ncols, nrows):
+        self._check(self._lib.galois_hip_f32_to_f16_panel(self._ctx, _ptr(x), _ptr(panel), ncols, nrows))
+
+    def rms_norm_mul_f16_panel(self, x, weight, panel, ncols, nrows, eps):
+        self._check(self._lib.galois_hip_rms_norm_mul_f16_panel(self._ctx, _ptr(x), _ptr(weight), _ptr(panel), ncols,
+                                                                nrows, eps))
+
+    def silu_mul_f16_panel(self, gate, up, panel, ncols, nrows):
+        self._check(self._lib.galois_hip_silu_mul_f16_panel(self._ctx, _ptr(gate), _ptr(up), _ptr(panel), ncols, nrows))
+
+    def mul_mat_q4_0_f16_panel(self, items, panel, K, M):
+        """items: [(W, Y, N), ...] (1 to 4 matrices against the same panel, one launch)."""
+        arr = (_abi.GemmItem * len(items))()
+        for a, (w, y, n) in zip(arr, items):
+            a.W, a.Y, a.N = _ptr(w), _ptr(y), n
+        self._check(self._lib.galois_hip_mul_mat_q4_0_f16_panel(self._ctx, arr, len(items), _ptr(panel), K, M))
+
     def rms_norm_f32(self, x, dst, ncols, nrows, eps):
         self._check(self._lib.galois_hip_rms_norm_f32(self._ctx, _ptr(x), _ptr(dst), ncols, nrows, eps))
 

@@ -21,6 +21,11 @@ class GemvItem(C.Structure):
                 ("scale_weight", vp), ("sumsq_out", vp), ("sumsq_in", vp)]
 
 
+class GemmItem(C.Structure):
+    """galois_hip_gemm_item of include/galois_hip.h, field for field."""
+    _fields_ = [("W", vp), ("Y", vp), ("N", i32), ("reserved", i32)]
+
+
 # name -> (restype, argtypes); must list every function the header declares
 PROTOTYPES = {
     "galois_hip_abi_version": (i32, []),
@@ -52,6 +57,11 @@ PROTOTYPES = {
     "galois_hip_dequantize_mul_mat_vec_q4_0": (i32, [c_ctx, vp, vp, vp, i32, i32]),
     "galois_hip_dequantize_mul_mat_vec_q4_0_group": (i32, [c_ctx, C.POINTER(GemvItem), i32]),
     "galois_hip_mul_mat_q4_0_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32]),
+    "galois_hip_f16_panel_bytes": (i32, [i32, i32, C.POINTER(C.c_int64)]),
+    "galois_hip_f32_to_f16_panel": (i32, [c_ctx, vp, vp, i32, i32]),
+    "galois_hip_rms_norm_mul_f16_panel": (i32, [c_ctx, vp, vp, vp, i32, i32, f32]),
+    "galois_hip_silu_mul_f16_panel": (i32, [c_ctx, vp, vp, vp, i32, i32]),
+    "galois_hip_mul_mat_q4_0_f16_panel": (i32, [c_ctx, C.POINTER(GemmItem), i32, vp, i32, i32]),
     "galois_hip_rms_norm_f32": (i32, [c_ctx, vp, vp, i32, i32, f32]),
     "galois_hip_rms_norm_mul_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, f32]),
     "galois_hip_rope_f32": (i32, [c_ctx, vp, vp, i32, i32, vp, f32, i32, f32]),

@@ -160,13 +160,16 @@ struct gemm_cfg {
 };
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-// X -> fp16 in the order the MFMA A operand is fetched: tiles of 16 rows x 32 k (1 KB), tile (m16, kb)
+// X -> fp16 in the order the MFMA A operand is fetched ("the panel"): tiles of 16 rows x 32 k (1 KB), tile (m16, kb)
 // at ((m16 * K/32) + kb) * 1 KB, and inside a tile the 16-byte run k = kb*32 + kg*8 .. +7 of row
 // m16*16 + r at (kg * 16 + r) * 16 bytes.  Lane l = kg * 16 + r of a wave owns exactly that run in
 // v_mfma_f32_16x16x32_f16, so a fragment load is 64 consecutive 16-byte pieces: one contiguous KB.
 // Rows past M (the last tile of a ragged M) are written as zeros.
-__global__ __launch_bounds__(256) void f32_to_f16_tiles(const float *__restrict__ x, _Float16 *__restrict__ y, int M,
-                                                        int K, int64_t nchunks) {
+// SWIGLU: the panel receives silu(x) * up instead of x (silu_f32 then mul_f32, unary.cu:1-10, mul.cu:3-12, with the
+// arithmetic of galois_hip_silu_mul_f32), so that a down projection needs neither that launch nor the conversion.
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void f32_to_f16_tiles(const float *__restrict__ x, const float *__restrict__ up,
+                                                        _Float16 *__restrict__ y, int M, int K, int64_t nchunks) {
     const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte output chunk
     if (o >= nchunks) return;
     const int64_t tile = o >> 6;
@@ -178,10 +181,80 @@ __global__ __launch_bounds__(256) void f32_to_f16_tiles(const float *__restrict_
     uint4 out = make_uint4(0, 0, 0, 0);
     if (m < M) {
         const float4 *src = reinterpret_cast<const float4 *>(x + m * K + kb * 32 + kg * 8);
-        const float4 a = src[0], b = src[1];
+        float4 a = src[0], b = src[1];
+        if (SWIGLU) {
+            const float4 *us = reinterpret_cast<const float4 *>(up + m * K + kb * 32 + kg * 8);
+            const float4 ua = us[0], ub = us[1];
+            a = make_float4(a.x / (1.0f + expf(-a.x)) * ua.x, a.y / (1.0f + expf(-a.y)) * ua.y,
+                            a.z / (1.0f + expf(-a.z)) * ua.z, a.w / (1.0f + expf(-a.w)) * ua.w);
+            b = make_float4(b.x / (1.0f + expf(-b.x)) * ub.x, b.y / (1.0f + expf(-b.y)) * ub.y,
+                            b.z / (1.0f + expf(-b.z)) * ub.z, b.w / (1.0f + expf(-b.w)) * ub.w);
+        }
         out.x = pack_h2(a.x, a.y), out.y = pack_h2(a.z, a.w), out.z = pack_h2(b.x, b.y), out.w = pack_h2(b.z, b.w);
     }
     reinterpret_cast<uint4 *>(y)[o] = out;
+}
+
+// rms_norm(x, eps) * weight (rms_norm.cu:13-49 then mul.cu:3-12) written straight into the panel: one workgroup per
+// row, the row in registers (NV runs of eight values per thread), the arithmetic of galois_hip_rms_norm_mul_f32
+// ((x * scale) * weight, rounded to fp16 at the end).  A thread's run is one 16-byte piece of the panel; the sixteen
+// rows of a tile group are given to workgroups of one XCD (blockIdx % 8), so that the pieces of a line meet in
+// one L2 before they are written back.
+constexpr int kPanelNormThreads = 512;
+template <int NV>
+__global__ __launch_bounds__(kPanelNormThreads) void rms_norm_to_f16_tiles(const float *__restrict__ x,
+                                                                            const float *__restrict__ w,
+                                                                            _Float16 *__restrict__ y, int M, int K, float eps,
+                                                                            int groups, int groups_per_xcd) {
+    constexpr int THREADS = kPanelNormThreads;
+    __shared__ float part[THREADS / 64];
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int grp = xcd * groups_per_xcd + (j >> 4), r = j & 15;
+    if (grp >= groups) return;
+    const int m = grp * 16 + r;
+    const bool live = m < M;  // rows past M are zeros in the panel
+    const int nrun = K >> 3;
+    float4 v[NV][2], g[NV][2];
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = threadIdx.x + i * THREADS;
+        const bool ok = live && c < nrun;
+        const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)(live ? m : 0) * K) + 2 * (ok ? c : 0);
+        v[i][0] = ok ? src[0] : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[i][1] = ok ? src[1] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = min(threadIdx.x + i * THREADS, nrun - 1);
+        g[i][0] = reinterpret_cast<const float4 *>(w)[2 * c];
+        g[i][1] = reinterpret_cast<const float4 *>(w)[2 * c + 1];
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            ss += v[i][h].x * v[i][h].x + v[i][h].y * v[i][h].y + v[i][h].z * v[i][h].z + v[i][h].w * v[i][h].w;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < THREADS / 64; i++) tot += part[i];
+    const float scale = 1.0f / sqrtf(tot / (float)K + eps);
+    const size_t tile_row = (size_t)grp * (K >> 5);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = threadIdx.x + i * THREADS;
+        if (c < nrun) {
+            const float4 a = v[i][0], b = v[i][1], ga = g[i][0], gb = g[i][1];
+            uint4 out;
+            out.x = pack_h2((a.x * scale) * ga.x, (a.y * scale) * ga.y), out.y = pack_h2((a.z * scale) * ga.z, (a.w * scale) * ga.w);
+            out.z = pack_h2((b.x * scale) * gb.x, (b.y * scale) * gb.y), out.w = pack_h2((b.z * scale) * gb.z, (b.w * scale) * gb.w);
+            reinterpret_cast<uint4 *>(y)[(tile_row + (c >> 2)) * 64 + (c & 3) * 16 + r] = out;
+        }
+    }
 }
 
 // Four nibble bytes (one dword of qs) -> 4 + 4 fp16 weights:
@@ -217,20 +290,55 @@ __device__ __forceinline__ void gload16(u32x4_t &dst, const void *ptr) {
 }
 #define GEMM_VMWAIT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
 
+// Up to GEMM_MAX_MATS weight matrices against the same panel in one launch (q | k | v, gate | up).  Their rows (the
+// columns of the results) are numbered through as one concatenated matrix and tiled as such -- a tile may end in one
+// matrix and go on in the next -- so three matrices of 4096 rows are exactly 128 tiles of 96 columns per 256-row
+// panel: 256 workgroups at M = 512, where each of them alone has 86 (or 172 of 48 columns) for 256 CUs.
+constexpr int GEMM_MAX_MATS = 4;
+struct gemm_mats {
+    const uint8_t *W[GEMM_MAX_MATS];
+    float *Y[GEMM_MAX_MATS];
+    int32_t N[GEMM_MAX_MATS];
+    int32_t col0[GEMM_MAX_MATS];  // first concatenated column of each matrix; unused entries hold INT_MAX
+    int32_t n_total;              // columns of the concatenation
+};
+
+// Row `c` of the concatenated weights (clamped to the last one): its bytes.
+__device__ __forceinline__ const uint8_t *gemm_w_row(const gemm_mats &mats, int c, size_t wrow_bytes) {
+    c = min(c, mats.n_total - 1);
+    const uint8_t *W = mats.W[0];
+    int first = 0;
+#pragma unroll
+    for (int j = 1; j < GEMM_MAX_MATS; j++) {
+        const bool ge = c >= mats.col0[j];
+        W = ge ? mats.W[j] : W, first = ge ? mats.col0[j] : first;
+    }
+    return W + (size_t)(c - first) * wrow_bytes;
+}
+
 template <int GN>
 struct gemm_raw_regs {
     u32x4_t c[gemm_cfg<GN>::RAW_PER_THREAD];
 };
 
+// rowp[i]: where the thread's i-th 16-byte chunk of a piece lies in the first piece of its weight row (the row and
+// the chunk are the same for every piece, so the matrix lookup happens once).
 template <int GN>
-__device__ __forceinline__ void gemm_load_raw(const uint8_t *W, size_t wrow_bytes, int N, int n0, int p, int super,
-                                              gemm_raw_regs<GN> &r) {
+__device__ __forceinline__ void gemm_raw_rows(const gemm_mats &mats, size_t wrow_bytes, int n0, int p,
+                                              const uint8_t *(&rowp)[gemm_cfg<GN>::RAW_PER_THREAD]) {
 #pragma unroll
     for (int i = 0; i < gemm_cfg<GN>::RAW_PER_THREAD; i++) {
         const int q = min(p + 256 * i, gemm_cfg<GN>::RAW_CHUNKS - 1);
         const int row = q / 9, c = q - row * 9;
-        gload16(r.c[i], W + (size_t)min(n0 + row, N - 1) * wrow_bytes + (size_t)super * GRAW_STRIDE + c * 16);
+        rowp[i] = gemm_w_row(mats, n0 + row, wrow_bytes) + c * 16;
     }
+}
+
+template <int GN>
+__device__ __forceinline__ void gemm_load_raw(const uint8_t *const (&rowp)[gemm_cfg<GN>::RAW_PER_THREAD], int super,
+                                              gemm_raw_regs<GN> &r) {
+#pragma unroll
+    for (int i = 0; i < gemm_cfg<GN>::RAW_PER_THREAD; i++) gload16(r.c[i], rowp[i] + (size_t)super * GRAW_STRIDE);
 }
 
 template <int GN>
@@ -295,7 +403,7 @@ __device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs<GN> &r, _
 // Barrier protocol (both kinds of wave meet every one): R after the first raw piece is parked,
 // then barrier t after stage t is written, for t = 0 .. nslots-1.  Stage t goes to buffer t % 3.
 template <int GN>
-__device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__restrict__ W, int K, int N, int n0) {
+__device__ __forceinline__ void gemm_producer(_Float16 *smem, const gemm_mats &mats, int K, int n0) {
     constexpr int GB_HALFS = gemm_cfg<GN>::B_HALFS, GRAW_BYTES = gemm_cfg<GN>::RAW_BYTES;
     const int p = threadIdx.x - 256;
     const int nslots = K / 64;            // stages; a multiple of 4 (K % 256 == 0)
@@ -305,10 +413,12 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
     uint8_t *raw1 = raw0 + GRAW_BYTES;
 
     gemm_raw_regs<GN> rr;
-    gemm_load_raw(W, wrow_bytes, N, n0, p, 0, rr);
+    const uint8_t *rowp[gemm_cfg<GN>::RAW_PER_THREAD];
+    gemm_raw_rows<GN>(mats, wrow_bytes, n0, p, rowp);
+    gemm_load_raw<GN>(rowp, 0, rr);
     GEMM_VMWAIT(0);
     gemm_store_raw(raw0, p, rr);
-    gemm_load_raw(W, wrow_bytes, N, n0, p, min(1, nsuper - 1), rr);
+    gemm_load_raw<GN>(rowp, min(1, nsuper - 1), rr);
     __syncthreads();  // R
     gemm_stage_regs<GN> s0, s1;
     gemm_stage_read<0>(s0, raw0, p);
@@ -328,7 +438,7 @@ __device__ __forceinline__ void gemm_producer(_Float16 *smem, const uint8_t *__r
         // passed a barrier three stages ago, and request the one after it
         GEMM_VMWAIT(0);
         gemm_store_raw(other, p, rr);
-        gemm_load_raw(W, wrow_bytes, N, n0, p, min(sup + 2, nsuper - 1), rr);
+        gemm_load_raw<GN>(rowp, min(sup + 2, nsuper - 1), rr);
         __syncthreads();
         gemm_stage_read<0>(s0, other, p);  // the next piece's first stage (read again, unused, after the last piece)
         gemm_stage_write(s1, smem + ((t + 3) % GNBUF) * GB_HALFS, p);
@@ -371,8 +481,7 @@ __device__ __forceinline__ void gemm_load_a1(u32x4_t &dst, const _Float16 *xs, u
 #define GEMM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
 template <int NF, int GN>
 __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float16 *__restrict__ Xh,
-                                              float *__restrict__ Y, int K, int N, int M, int m0, int n0, int wm,
-                                              int ncol0) {
+                                              const gemm_mats &mats, int K, int M, int m0, int n0, int wm, int ncol0) {
     constexpr int GB_HALFS = gemm_cfg<GN>::B_HALFS;
     const int lane = threadIdx.x & 63;
     const int nslots = K / 64;
@@ -485,24 +594,32 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
         GEMM_DRAIN_A(a3);
     }
 
-    // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e
+    // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e.  A lane's column lies in one of the
+    // matrices of the launch: the result goes to that matrix's Y.
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int j = 0; j < NF; j++) {
+        const int n = n0 + ncol0 + j * 16 + (lane & 15);
+        float *Y = mats.Y[0];
+        int N = mats.N[0], first = 0;
 #pragma unroll
-        for (int j = 0; j < NF; j++) {
-            const int n = n0 + ncol0 + j * 16 + (lane & 15);
+        for (int t = 1; t < GEMM_MAX_MATS; t++) {
+            const bool ge = n >= mats.col0[t];
+            Y = ge ? mats.Y[t] : Y, N = ge ? mats.N[t] : N, first = ge ? mats.col0[t] : first;
+        }
+        const int nl = n - first;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + e;
-                if (m < M && n < N) Y[(size_t)m * N + n] = acc[i][j][e];
+                if (m < M && n < mats.n_total) Y[(size_t)m * N + nl] = acc[i][j][e];
             }
-        }
+    }
 }
 
 template <int GN>
-__global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict__ W, const _Float16 *__restrict__ Xh,
-                                                      float *__restrict__ Y, int K, int N, int M, int n_tiles,
-                                                      int m_tiles) {
+__global__ __launch_bounds__(512) void gemm_q4_0_mfma(const gemm_mats mats, const _Float16 *__restrict__ Xh, int K, int M,
+                                                      int n_tiles, int m_tiles) {
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[];  // [3] B stage | [2] raw | pad
     // XCD-aware tile order: blockIdx % 8 is the XCD; consecutive tiles (same X panel) go to one XCD
     const int total = n_tiles * m_tiles;
@@ -513,15 +630,16 @@ __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const uint8_t *__restrict_
     const int m0 = mt * GM, n0 = nt * GN;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (wave >= 4)
-        gemm_producer<GN>(smem, W, K, N, n0);
+        gemm_producer<GN>(smem, mats, K, n0);
     else  // four consumer waves stacked in M, each 64 rows x GN columns
-        gemm_consumer<GN / 16, GN>(smem, Xh, Y, K, N, M, m0, n0, wave, 0);
+        gemm_consumer<GN / 16, GN>(smem, Xh, mats, K, M, m0, n0, wave, 0);
 }
 
 // Launch of one tile width.
 template <int GN>
-int32_t gemm_launch(galois_hip_ctx *ctx, const uint8_t *W, const _Float16 *Xh, float *Y, int K, int N, int M) {
-    const int n_tiles = (N + GN - 1) / GN, m_tiles = (M + GM - 1) / GM;
+int32_t gemm_launch(galois_hip_ctx *ctx, const gemm_mats &mats, const _Float16 *Xh, int K, int M) {
+    const int n_tiles = (mats.n_total + GN - 1) / GN;
+    const int m_tiles = (M + GM - 1) / GM;
     const int total = n_tiles * m_tiles;
     const int grid = ((total + 7) / 8) * 8;
     const size_t lds = gemm_cfg<GN>::LDS_BYTES;
@@ -529,7 +647,39 @@ int32_t gemm_launch(galois_hip_ctx *ctx, const uint8_t *W, const _Float16 *Xh, f
     // for every device and every thread without any flag of our own
     hipError_t e = hipFuncSetAttribute((const void *)gemm_q4_0_mfma<GN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
-    hipLaunchKernelGGL(gemm_q4_0_mfma<GN>, dim3(grid), dim3(512), lds, ctx->stream, W, Xh, Y, K, N, M, n_tiles, m_tiles);
+    hipLaunchKernelGGL(gemm_q4_0_mfma<GN>, dim3(grid), dim3(512), lds, ctx->stream, mats, Xh, K, M, n_tiles, m_tiles);
+    return GALOIS_HIP_OK;
+}
+
+// Tile width by how many workgroups it gives the device.  Cost model: rounds of workgroups over the CUs
+// times the relative cost of a k-stage (a 48-column stage has half the matrix instructions and half
+// the dequantisation of a 96-column one but the same barriers and A requests: ~0.65).
+int32_t gemm_launch_any(galois_hip_ctx *ctx, gemm_mats mats, int n_mats, const _Float16 *Xh, int K, int M) {
+    int64_t cols = 0;
+    for (int j = 0; j < GEMM_MAX_MATS; j++) {
+        mats.col0[j] = j < n_mats ? (int32_t)cols : 0x7FFFFFFF;
+        if (j < n_mats) cols += mats.N[j];
+    }
+    mats.n_total = (int32_t)cols;
+    const int64_t m_tiles = (M + GM - 1) / GM;
+    const int64_t wg96 = (cols + 95) / 96 * m_tiles, wg48 = (cols + 47) / 48 * m_tiles;
+    const int64_t cus = ctx->n_cu > 0 ? ctx->n_cu : 256;
+    const double cost96 = (double)((wg96 + cus - 1) / cus), cost48 = 0.65 * (double)((wg48 + cus - 1) / cus);
+    return cost48 < cost96 ? gemm_launch<48>(ctx, mats, Xh, K, M) : gemm_launch<96>(ctx, mats, Xh, K, M);
+}
+
+// What the main kernel asks of its operands: whole 4-stage pieces of every weight row, 16-byte requests, and a panel
+// whose byte offsets fit 32 bits.
+bool gemm_panel_shape_ok(int64_t K, int64_t M) { return K > 0 && M > 0 && K % 256 == 0 && (M + 16) * K * 2 < ((int64_t)1 << 32); }
+
+int32_t launch_to_panel(galois_hip_ctx *ctx, const float *x, const float *up, _Float16 *panel, int K, int M, bool swiglu) {
+    const int64_t m_pad = ((int64_t)M + 15) / 16 * 16;
+    const int64_t nchunks = m_pad * K / 8;
+    const dim3 grid((unsigned)((nchunks + 255) / 256)), block(256);
+    if (swiglu)
+        hipLaunchKernelGGL(f32_to_f16_tiles<true>, grid, block, 0, ctx->stream, x, up, panel, M, K, nchunks);
+    else
+        hipLaunchKernelGGL(f32_to_f16_tiles<false>, grid, block, 0, ctx->stream, x, up, panel, M, K, nchunks);
     return GALOIS_HIP_OK;
 }
 
@@ -544,7 +694,7 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
     GH_REQUIRE(ctx, gh_aligned(W, 2) && gh_aligned(X, 16) && gh_aligned(Y, 4), GALOIS_HIP_E_ALIGN,
                "mul_mat_q4_0_f32: W 2-byte, X 16-byte, Y 4-byte aligned");
     GH_BIND(ctx);
-    if (K % 256 == 0 && gh_aligned(W, 16) && ((int64_t)M + 16) * K * 2 < ((int64_t)1 << 32)) {
+    if (gemm_panel_shape_ok(K, M) && gh_aligned(W, 16)) {
         // fp16 copy of X, tiled for the A fragments, in the context's workspace (grown on demand)
         const int64_t m_pad = ((int64_t)M + 15) / 16 * 16;
         const size_t need = (size_t)m_pad * K * sizeof(_Float16);
@@ -561,23 +711,97 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
             ctx->ws_bytes = bytes;
         }
         _Float16 *Xh = (_Float16 *)ctx->ws;
-        const int64_t nchunks = m_pad * K / 8;
-        hipLaunchKernelGGL(f32_to_f16_tiles, dim3((unsigned)((nchunks + 255) / 256)), dim3(256), 0, ctx->stream, X, Xh, M,
-                           K, nchunks);
-        // Tile width by how many workgroups it gives the device.  Cost model: rounds of workgroups over the CUs
-        // times the relative cost of a k-stage (a 48-column stage has half the matrix instructions and half
-        // the dequantisation of a 96-column one but the same barriers and A requests: ~0.65).
-        const int64_t m_tiles = (M + GM - 1) / GM;
-        const int64_t wg96 = (N + 95) / 96 * m_tiles, wg48 = (N + 47) / 48 * m_tiles;
-        const int64_t cus = ctx->n_cu > 0 ? ctx->n_cu : 256;
-        const double cost96 = (double)((wg96 + cus - 1) / cus), cost48 = 0.65 * (double)((wg48 + cus - 1) / cus);
-        int tile_n = cost48 < cost96 ? 48 : 96;
-        const int32_t st = tile_n == 48 ? gemm_launch<48>(ctx, (const uint8_t *)W, Xh, Y, K, N, M)
-                                        : gemm_launch<96>(ctx, (const uint8_t *)W, Xh, Y, K, N, M);
+        launch_to_panel(ctx, X, nullptr, Xh, K, M, false);
+        gemm_mats mats = {};
+        mats.W[0] = (const uint8_t *)W, mats.Y[0] = Y, mats.N[0] = N;
+        const int32_t st = gemm_launch_any(ctx, mats, 1, Xh, K, M);
         if (st != GALOIS_HIP_OK) return st;
     } else {
         const dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
         hipLaunchKernelGGL(gemm_q4_0_mfma_v1, grid, dim3(256), 0, ctx->stream, (const uint8_t *)W, X, Y, K, N, M);
     }
     GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f32 launch");
+}
+
+// ---- the panel as an operand of its own: producers that write it, and the matmul that takes it ----
+
+extern "C" int32_t galois_hip_f16_panel_bytes(int32_t K, int32_t M, int64_t *bytes) {
+    if (!bytes) return GALOIS_HIP_E_NULL;
+    *bytes = 0;
+    if (!gemm_panel_shape_ok(K, M)) return GALOIS_HIP_E_SHAPE;
+    *bytes = ((int64_t)M + 15) / 16 * 16 * K * (int64_t)sizeof(_Float16);
+    return GALOIS_HIP_OK;
+}
+
+static int32_t panel_args(galois_hip_ctx *ctx, const void *a, const void *b, const void *panel, int32_t K, int32_t M,
+                          const char *what) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, a && b && panel, GALOIS_HIP_E_NULL, what);
+    GH_REQUIRE(ctx, gemm_panel_shape_ok(K, M), GALOIS_HIP_E_SHAPE,
+               "f16 panel: ncols a positive multiple of 256, nrows positive, (nrows + 16) * ncols below 2^31");
+    GH_REQUIRE(ctx, gh_aligned(a, 16) && gh_aligned(b, 16) && gh_aligned(panel, 16), GALOIS_HIP_E_ALIGN,
+               "f16 panel: 16-byte aligned operands");
+    return GALOIS_HIP_OK;
+}
+
+extern "C" int32_t galois_hip_f32_to_f16_panel(galois_hip_ctx *ctx, const float *x, void *panel, int32_t ncols, int32_t nrows) {
+    const int32_t st = panel_args(ctx, x, x, panel, ncols, nrows, "f32_to_f16_panel");
+    if (st != GALOIS_HIP_OK) return st;
+    GH_BIND(ctx);
+    launch_to_panel(ctx, x, nullptr, (_Float16 *)panel, ncols, nrows, false);
+    GH_LAUNCH_CHECK(ctx, "f32_to_f16_panel launch");
+}
+
+extern "C" int32_t galois_hip_silu_mul_f16_panel(galois_hip_ctx *ctx, const float *gate, const float *up, void *panel,
+                                                 int32_t ncols, int32_t nrows) {
+    const int32_t st = panel_args(ctx, gate, up, panel, ncols, nrows, "silu_mul_f16_panel");
+    if (st != GALOIS_HIP_OK) return st;
+    GH_BIND(ctx);
+    launch_to_panel(ctx, gate, up, (_Float16 *)panel, ncols, nrows, true);
+    GH_LAUNCH_CHECK(ctx, "silu_mul_f16_panel launch");
+}
+
+extern "C" int32_t galois_hip_rms_norm_mul_f16_panel(galois_hip_ctx *ctx, const float *x, const float *weight, void *panel,
+                                                     int32_t ncols, int32_t nrows, float eps) {
+    const int32_t st = panel_args(ctx, x, weight, panel, ncols, nrows, "rms_norm_mul_f16_panel");
+    if (st != GALOIS_HIP_OK) return st;
+    const int nv = (ncols / 8 + kPanelNormThreads - 1) / kPanelNormThreads;
+    GH_REQUIRE(ctx, nv <= 4, GALOIS_HIP_E_SHAPE, "rms_norm_mul_f16_panel: rows of at most 16384 columns");
+    GH_BIND(ctx);
+    const int groups = (nrows + 15) / 16, per_xcd = (groups + 7) / 8;
+    const dim3 grid((unsigned)(8 * per_xcd * 16)), block(kPanelNormThreads);
+    _Float16 *y = (_Float16 *)panel;
+    if (nv <= 1)
+        hipLaunchKernelGGL(rms_norm_to_f16_tiles<1>, grid, block, 0, ctx->stream, x, weight, y, nrows, ncols, eps, groups, per_xcd);
+    else if (nv <= 2)
+        hipLaunchKernelGGL(rms_norm_to_f16_tiles<2>, grid, block, 0, ctx->stream, x, weight, y, nrows, ncols, eps, groups, per_xcd);
+    else
+        hipLaunchKernelGGL(rms_norm_to_f16_tiles<4>, grid, block, 0, ctx->stream, x, weight, y, nrows, ncols, eps, groups, per_xcd);
+    GH_LAUNCH_CHECK(ctx, "rms_norm_mul_f16_panel launch");
+}
+
+extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel(galois_hip_ctx *ctx, const galois_hip_gemm_item *items, int32_t n_items,
+                                                     const void *panel, int32_t K, int32_t M) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, items && panel, GALOIS_HIP_E_NULL, "mul_mat_q4_0_f16_panel");
+    GH_REQUIRE(ctx, n_items >= 1 && n_items <= GEMM_MAX_MATS, GALOIS_HIP_E_SHAPE, "mul_mat_q4_0_f16_panel: 1 to 4 matrices per call");
+    GH_REQUIRE(ctx, gemm_panel_shape_ok(K, M), GALOIS_HIP_E_SHAPE,
+               "mul_mat_q4_0_f16_panel: K a positive multiple of 256, M positive, (M + 16) * K below 2^31");
+    GH_REQUIRE(ctx, gh_aligned(panel, 16), GALOIS_HIP_E_ALIGN, "mul_mat_q4_0_f16_panel: 16-byte aligned panel");
+    gemm_mats mats = {};
+    int64_t cols = 0;
+    for (int j = 0; j < n_items; j++) {
+        GH_REQUIRE(ctx, items[j].W && items[j].Y, GALOIS_HIP_E_NULL, "mul_mat_q4_0_f16_panel");
+        GH_REQUIRE(ctx, items[j].N > 0, GALOIS_HIP_E_SHAPE, "mul_mat_q4_0_f16_panel: N positive");
+        GH_REQUIRE(ctx, gh_aligned(items[j].W, 16) && gh_aligned(items[j].Y, 4), GALOIS_HIP_E_ALIGN,
+                   "mul_mat_q4_0_f16_panel: W 16-byte, Y 4-byte aligned");
+        mats.W[j] = (const uint8_t *)items[j].W, mats.Y[j] = items[j].Y, mats.N[j] = items[j].N;
+        cols += items[j].N;
+    }
+    GH_REQUIRE(ctx, cols < 0x7FFFFF00 && (cols + 47) / 48 * ((M + GM - 1) / GM) < 0x7FFFFF00, GALOIS_HIP_E_SHAPE,
+               "mul_mat_q4_0_f16_panel: too many columns");
+    GH_BIND(ctx);
+    const int32_t st = gemm_launch_any(ctx, mats, n_items, (const _Float16 *)panel, K, M);
+    if (st != GALOIS_HIP_OK) return st;
+    GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel launch");
 }

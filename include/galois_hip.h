@@ -34,7 +34,7 @@ extern "C" {
 #endif
 
 /* Changes whenever the argument list of an exported function changes (2: n_table_rows of get_rows_q4_0,
- * head_major_n_ctx of the attention calls, galois_hip_abi_version / galois_hip_set_option added).  A binding compares
+ * head_major_n_ctx of the attention calls, galois_hip_abi_version / galois_hip_set_option and the panel calls added).  A binding compares
  * the value it was written against with galois_hip_abi_version() before its first call. */
 #define GALOIS_HIP_ABI_VERSION 2
 
@@ -198,6 +198,39 @@ int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *ctx, const 
 int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *W, const float *X, float *Y,
                                     int32_t K, int32_t N, int32_t M);
 
+/* The prefill matmul on activations that are ALREADY in the form its matrix instructions fetch ("the panel": fp16,
+ * tiles of 16 rows x 32 columns, 1 KB each, tile (r16, c32) at (r16 * K/32 + c32) KB, inside a tile the eight
+ * consecutive values k = c32*32 + g*8 .. of row r16*16 + r at (g * 16 + r) * 16 bytes; rows past M are zero), and
+ * the producers that write it.  No counterpart in the reference, whose quantize_q8_1 pass (src/cuda.rs:1066-1087 ->
+ * matmul.cu:133-174) runs inside every matmul call: galois_hip_mul_mat_q4_0_f32 likewise converts X on every call
+ * (one launch, 5-6 us at 512 x 4096); a prefill graph that multiplies the same activations by several matrices
+ * (q | k | v after the attention norm, gate | up after the FFN norm), or whose activations come out of a norm or a
+ * SwiGLU anyway, writes the panel once, from the op that produces the activations, and hands it on:
+ *   galois_hip_f16_panel_bytes: size of the panel of an M x K activation matrix (K % 256 == 0);
+ *   galois_hip_f32_to_f16_panel: the conversion alone;
+ *   galois_hip_rms_norm_mul_f16_panel: rms_norm_f32 + mul_f32 (src/cuda.rs:1146-1215) with the arithmetic of
+ *     galois_hip_rms_norm_mul_f32, rounded to fp16 (nearest even) into the panel; ncols <= 16384;
+ *   galois_hip_silu_mul_f16_panel: silu_f32 + mul_f32 (src/cuda.rs:1665-1688, 1190-1215) likewise;
+ *   galois_hip_mul_mat_q4_0_f16_panel: Y_j[m*N_j + n] = sum_k deq(W_j)[n,k] * panel[m,k] for 1 to 4 matrices in ONE
+ *     launch, each what galois_hip_mul_mat_q4_0_f32 computes from the f32 activations the panel was rounded from
+ *     (bit for bit when the panel came from galois_hip_f32_to_f16_panel).  The matrices' column tiles are laid end to
+ *     end, so q | k | v of a 4096-wide model fill the device at M = 512 where each alone leaves a third of it idle.
+ *     W_j 16-byte aligned (rows of K/32 blocks), Y_j 4-byte, panel 16-byte aligned. */
+typedef struct galois_hip_gemm_item {
+    const void *W;
+    float *Y;
+    int32_t N;
+    int32_t reserved; /* 0 */
+} galois_hip_gemm_item;
+int32_t galois_hip_f16_panel_bytes(int32_t K, int32_t M, int64_t *bytes);
+int32_t galois_hip_f32_to_f16_panel(galois_hip_ctx *ctx, const float *x, void *panel, int32_t ncols, int32_t nrows);
+int32_t galois_hip_rms_norm_mul_f16_panel(galois_hip_ctx *ctx, const float *x, const float *weight, void *panel,
+                                          int32_t ncols, int32_t nrows, float eps);
+int32_t galois_hip_silu_mul_f16_panel(galois_hip_ctx *ctx, const float *gate, const float *up, void *panel,
+                                      int32_t ncols, int32_t nrows);
+int32_t galois_hip_mul_mat_q4_0_f16_panel(galois_hip_ctx *ctx, const galois_hip_gemm_item *items, int32_t n_items,
+                                          const void *panel, int32_t K, int32_t M);
+
 /* rms_norm_f32 launch, src/cuda.rs:1146-1181 -> rms_norm.cu:13-49:
  * dst = x * rsqrt(mean(x^2) + eps) per row.  Unlike the reference (ne00 % 32 == 0
  * asserted at src/cuda.rs:1157) any ncols >= 1 is accepted. */
@@ -261,7 +294,10 @@ int32_t galois_hip_mul_mat_f32(galois_hip_ctx *ctx, const float *a, const float 
  * reference serves with cuBLAS gemm_ex on f16 operands with f16 accumulation and an f16 result
  * (CudaMatMul::f_x_y_y, src/cuda.rs:881-992 -> cuda_op_mul_mat_cublas, src/cuda.rs:698-757).  Here a is widened
  * exactly and sums are f32; with M > 1 and rows of a contiguous along K (K % 32 == 0, 16-byte aligned rows) the
- * product runs on the matrix cores with b rounded to f16 as the reference's convert_fp32_to_fp16 does. */
+ * product runs on the matrix cores with b rounded to f16 as the reference's convert_fp32_to_fp16 does (|b| above
+ * 65504 becomes infinite there).  Everywhere else -- M == 1, K % 32 != 0, unaligned rows, a read along N -- b stays
+ * f32, so the same operands multiplied at M == 1 (decode) and at M > 1 (prefill) differ by that rounding: at most
+ * 2^-11 relative per element of b. */
 int32_t galois_hip_mul_mat_f16_f32(galois_hip_ctx *ctx, const void *a, const float *b, float *dst, int32_t K, int32_t N,
                                    int32_t M, int32_t ne02, int32_t ne12, int64_t a_s0, int64_t a_s1, int64_t a_s2);
 

@@ -1,0 +1,146 @@
+"""The prefill matmul on an fp16 panel (activations already in the order the matrix instructions fetch them) and the
+ops that write the panel, through the C ABI.
+
+Bars: the panel written by galois_hip_f32_to_f16_panel is the f32 matrix rounded to fp16 (numpy's nearest-even), tile
+for tile; a matmul on it equals galois_hip_mul_mat_q4_0_f32 on the f32 matrix bit for bit, alone or as one of several
+matrices in a launch; the norm and SwiGLU producers hold fp16(their f32 op) up to one unit in the last place of fp16
+(their reductions and exponentials round like the f32 ops', whose results the oracle gives to 1e-6), and the product
+on their panels is within the prefill bar (2e-3) of the oracle's f64 dequantize-then-GEMM on the oracle's activations.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from tests import npref
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def _untile(raw, m, k):
+    """Panel bytes -> [m_pad, k] float16: tile (r16, c32) is 1 KB, its 16-byte piece (g, r) holds columns c32*32 + g*8 .."""
+    m_pad = (m + 15) // 16 * 16
+    t = raw.view(np.float16).reshape(m_pad // 16, k // 32, 4, 16, 8)
+    return t.transpose(0, 3, 1, 2, 4).reshape(m_pad, k)
+
+
+def _panel(dev, k, m):
+    n = dev.f16_panel_bytes(k, m)
+    assert n == (m + 15) // 16 * 16 * k * 2
+    return dev.alloc(n), n
+
+
+def _case(seed, m, k, ns):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wqs = [oracle.quantize_q4_0((rng.standard_normal((n, k)) * 0.02).astype(np.float32)) for n in ns]
+    return x, wqs
+
+
+@pytest.mark.parametrize("m,k", [(512, 4096), (130, 256), (1, 512), (17, 11008)])
+def test_the_panel_is_the_matrix_rounded_to_fp16(dev, m, k):
+    x, _ = _case(m + k, m, k, [])
+    xb = dev.upload(x)
+    pb, nbytes = _panel(dev, k, m)
+    dev.upload(np.full(nbytes // 4, 7.5, np.float32), pb)
+    dev.f32_to_f16_panel(xb, pb, k, m)
+    got = _untile(dev.download(pb, np.uint8, nbytes), m, k)
+    assert np.array_equal(got[:m].view(np.uint16), x.astype(np.float16).view(np.uint16))
+    assert np.all(got[m:] == 0), "rows past M are zero"
+    for b in (xb, pb):
+        dev.free(b)
+
+
+@pytest.mark.parametrize("m,k,ns", [(512, 4096, [4096, 4096, 4096]), (512, 4096, [11008, 11008]), (512, 4096, [11008]),
+                                    (130, 256, [100, 4096, 177, 48]), (300, 1024, [96, 97]), (16, 2048, [5000])])
+def test_matmul_on_the_panel_equals_the_f32_call_bit_for_bit(dev, m, k, ns):
+    x, wqs = _case(m * 3 + k + len(ns), m, k, ns)
+    xb = dev.upload(x)
+    wbs = [dev.upload(w) for w in wqs]
+    pb, _ = _panel(dev, k, m)
+    dev.f32_to_f16_panel(xb, pb, k, m)
+    ys = [dev.alloc((m * n + 16) * 4) for n in ns]
+    for y, n in zip(ys, ns):
+        dev.upload(np.full(m * n + 16, 7.5, np.float32), y)
+    print("panel matmul m=%d k=%d ns=%s" % (m, k, ns), flush=True)
+    dev.mul_mat_q4_0_f16_panel([(w, y, n) for w, y, n in zip(wbs, ys, ns)], pb, k, m)
+    ref = dev.alloc(m * max(ns) * 4)
+    for w, wq, y, n in zip(wbs, wqs, ys, ns):
+        got = dev.download(y, np.float32, m * n + 16)
+        assert np.all(got[m * n:] == 7.5), "wrote past the end of Y"
+        dev.mul_mat_q4_0_f32(w, xb, ref, k, n, m)
+        one = dev.download(ref, np.float32, m * n)
+        assert np.array_equal(got[:m * n].view(np.uint32), one.view(np.uint32)), n
+        cols = np.unique(np.concatenate([[0, n - 1], np.random.default_rng(n).choice(n, min(n, 64), replace=False)]))
+        emax, el2 = npref.rel_err(got[:m * n].reshape(m, n)[:, cols], oracle.mul_mat_q4_0_f32(wq[cols], x))
+        assert emax < TOL and el2 < TOL, (n, emax, el2)
+    for b in [xb, pb, ref] + wbs + ys:
+        dev.free(b)
+
+
+def _ulps_f16(a, b):
+    """Largest distance between two float16 arrays in units of the last place of the larger magnitude."""
+    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+    ulp = np.maximum(np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32), 2.0 ** -24)
+    return float(np.max(np.abs(a32 - b32) / ulp))
+
+
+@pytest.mark.parametrize("m,k,n", [(512, 4096, 4096), (130, 256, 200), (33, 11008, 96), (5, 16384, 64)])
+def test_rms_norm_into_the_panel(dev, m, k, n):
+    rng = np.random.default_rng(m + k)
+    x = (rng.standard_normal((m, k)) * rng.uniform(0.1, 4.0, (m, 1))).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    wq = oracle.quantize_q4_0((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    xb, gb, wb, yb = dev.upload(x), dev.upload(g), dev.upload(wq), dev.alloc(m * n * 4)
+    pb, nbytes = _panel(dev, k, m)
+    dev.upload(np.full(nbytes // 4, 7.5, np.float32), pb)
+    dev.rms_norm_mul_f16_panel(xb, gb, pb, k, m, 1e-6)
+    act = oracle.mul(oracle.rms_norm(x, 1e-6), g)
+    got = _untile(dev.download(pb, np.uint8, nbytes), m, k)
+    assert np.all(got[m:] == 0)
+    assert _ulps_f16(got[:m], act.astype(np.float16)) <= 1.0
+    dev.mul_mat_q4_0_f16_panel([(wb, yb, n)], pb, k, m)
+    emax, el2 = npref.rel_err(dev.download(yb, np.float32, (m, n)), oracle.mul_mat_q4_0_f32(wq, act))
+    assert emax < TOL and el2 < TOL, (emax, el2)
+    for b in (xb, gb, wb, yb, pb):
+        dev.free(b)
+
+
+@pytest.mark.parametrize("m,k,n", [(512, 11008, 512), (130, 256, 200), (1, 768, 33)])
+def test_swiglu_into_the_panel(dev, m, k, n):
+    rng = np.random.default_rng(m * 5 + k)
+    gate = (rng.standard_normal((m, k)) * 2).astype(np.float32)
+    up = rng.standard_normal((m, k)).astype(np.float32)
+    wq = oracle.quantize_q4_0((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    gb, ub, wb, yb = dev.upload(gate), dev.upload(up), dev.upload(wq), dev.alloc(m * n * 4)
+    pb, nbytes = _panel(dev, k, m)
+    dev.silu_mul_f16_panel(gb, ub, pb, k, m)
+    act = oracle.mul(oracle.silu(gate).reshape(-1), up.reshape(-1)).reshape(m, k)
+    got = _untile(dev.download(pb, np.uint8, nbytes), m, k)
+    assert np.all(got[m:] == 0)
+    assert _ulps_f16(got[:m], act.astype(np.float16)) <= 1.0
+    dev.mul_mat_q4_0_f16_panel([(wb, yb, n)], pb, k, m)
+    emax, el2 = npref.rel_err(dev.download(yb, np.float32, (m, n)), oracle.mul_mat_q4_0_f32(wq, act))
+    assert emax < TOL and el2 < TOL, (emax, el2)
+    for b in (gb, ub, wb, yb, pb):
+        dev.free(b)
+
+
+def test_panel_argument_errors(dev):
+    from galois_amd import GaloisHipError
+    buf = dev.alloc(1 << 16)
+    with pytest.raises(GaloisHipError) as ei:
+        dev.f16_panel_bytes(100, 4)                        # K must be a multiple of 256
+    assert ei.value.status == -2
+    for call, code in ((lambda: dev.f32_to_f16_panel(buf, buf, 128, 4), -2),
+                       (lambda: dev.f32_to_f16_panel(buf.view(4), buf, 256, 4), -3),
+                       (lambda: dev.rms_norm_mul_f16_panel(buf, None, buf, 256, 4, 1e-6), -1),
+                       (lambda: dev.silu_mul_f16_panel(buf, buf, buf, 256, 0), -2),
+                       (lambda: dev.mul_mat_q4_0_f16_panel([], buf, 256, 4), -2),
+                       (lambda: dev.mul_mat_q4_0_f16_panel([(buf, buf, 8)] * 5, buf, 256, 4), -2),
+                       (lambda: dev.mul_mat_q4_0_f16_panel([(buf.view(2), buf, 8)], buf, 256, 4), -3),
+                       (lambda: dev.mul_mat_q4_0_f16_panel([(buf, buf, 0)], buf, 256, 4), -2)):
+        with pytest.raises(GaloisHipError) as ei:
+            call()
+        assert ei.value.status == code, (ei.value.status, code)
+    dev.free(buf)

@@ -72,6 +72,41 @@ def test_f16_weights_on_the_matrix_cores(dev, K, N, M, ne02, ne12):
         dev.free(x)
 
 
+def test_one_row_and_many_rows_of_the_same_operands_agree_within_the_stated_rounding(dev):
+    """The arm rounds b to f16 only where it runs on the matrix cores (M > 1, rows of a contiguous along K,
+    K % 32 == 0); one row of activations (decode) keeps b in f32.  The same row multiplied both ways therefore
+    differs by b's rounding and by nothing else: at most 2^-11 relative per element of b, i.e. within
+    2^-11 * sum |a| |b| element by element (1e-3 of the largest result on these operands); with activations that f16
+    holds exactly the two paths agree to the order of their f32 sums."""
+    rng = np.random.default_rng(17)
+    K, N, M = 4096, 512, 33
+    a = (rng.standard_normal((1, N, K)) * 0.05).astype(np.float16)
+    b = rng.standard_normal((1, M, K)).astype(np.float32)
+    ab, ob = dev.upload(a), dev.alloc(M * N * 4)
+
+    def both(bm):
+        bb = dev.upload(bm)
+        dev.mul_mat_f16_f32(ab, bb, ob, K, N, M, 1, 1, 1, K, N * K)            # M rows: matrix cores, b rounded to f16
+        many = dev.download(ob, np.float32, (M, N))
+        one = np.empty_like(many)
+        for r in range(M):                                                      # row by row: b stays f32
+            dev.mul_mat_f16_f32(ab, bb.view(r * K * 4), ob, K, N, 1, 1, 1, 1, K, N * K)
+            one[r] = dev.download(ob, np.float32, N)
+        dev.free(bb)
+        return many, one
+
+    many, one = both(b)
+    bound = 2.0 ** -11 * (np.abs(b[0]).astype(np.float64) @ np.abs(a[0].astype(np.float64)).T)
+    assert np.all(np.abs(many.astype(np.float64) - one) <= bound + 1e-5 * np.max(np.abs(one)))
+    emax, el2 = npref.rel_err(many, one)
+    assert emax < 1e-3 and el2 < 1e-3, (emax, el2)
+    many, one = both(b.astype(np.float16).astype(np.float32))                   # nothing left to round
+    emax, el2 = npref.rel_err(many, one)
+    assert emax < 1e-5 and el2 < 1e-5, (emax, el2)
+    for x in (ab, ob):
+        dev.free(x)
+
+
 def test_operands_the_matrix_core_kernel_does_not_take(dev):
     """K not a multiple of 32, or rows of a that are not 16-byte aligned: the generic kernels, exact widening."""
     rng = np.random.default_rng(5)
