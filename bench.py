@@ -61,8 +61,29 @@ def make_q4_matrix(dev, rng, k, n):
     return out
 
 
-def timed(dev, fn, iters, reps=1):
+SETTLE_S = 0.3   # every side measurement first runs its own launches for this long: after the idle time its set-up
+                 # leaves (uploads, allocations) the device needs ~0.25 s of work to be back at its steady clocks
+                 # (measured with rocm-smi: 1.4 -> 1.75 -> 1.9 -> 2.0 GHz over the first 0.3 s of a kernel loop), and a
+                 # hundred launches of a 4-10 us kernel are over long before that
+
+
+def settle(dev, fn, seconds=SETTLE_S):
+    """Runs fn(i) back to back for `seconds` of wall time (synchronising every 64 calls)."""
+    t_end = time.perf_counter() + seconds
+    i = 0
+    while time.perf_counter() < t_end:
+        fn(i)
+        i += 1
+        if i % 64 == 0:
+            dev.synchronize()
+    dev.synchronize()
+    return i
+
+
+def timed(dev, fn, iters, reps=1, settle_s=0.0):
     """Median over `reps` of the event-timed duration (ms) of `iters` calls of fn(i)."""
+    if settle_s:
+        settle(dev, fn, settle_s)
     e0, e1 = dev.event(), dev.event()
     out = []
     for _ in range(reps):
@@ -78,7 +99,7 @@ def timed(dev, fn, iters, reps=1):
     return float(np.median(out))
 
 
-def timed_graph(dev, fn, iters, reps=5):
+def timed_graph(dev, fn, iters, reps=5, settle_s=0.0):
     """As timed(), with the `iters` launches recorded once into a HIP graph and replayed: the figure for kernels
     short enough that issuing them one by one from Python is what an eager loop measures."""
     dev.synchronize()
@@ -88,6 +109,8 @@ def timed_graph(dev, fn, iters, reps=5):
     graph = dev.graph_end_capture()
     e0, e1 = dev.event(), dev.event()
     dev.graph_launch(graph)
+    if settle_s:
+        settle(dev, lambda i: dev.graph_launch(graph), settle_s)
     out = []
     for _ in range(reps):
         dev.synchronize()
@@ -177,6 +200,9 @@ def _normal_f32(seed, count, scale, threads=16):
     return out
 
 
+SETTLE_STEPS = 150   # decode steps (1.6-3 ms each) run before a plan is timed: the same settling as SETTLE_S
+
+
 def decode_step_bench(dev, reps, with_graph=True):
     """BASELINE.json configs[4]: a 32-layer LLaMA-7B-architecture decode step at KV length 2048, issued through the
     host mirror's galois ops, random-init weights quantized on the device.  Returns tokens/s three ways."""
@@ -238,7 +264,7 @@ def decode_step_bench(dev, reps, with_graph=True):
     for name, fused in (("eager_one_kernel_per_op", 0), ("eager_fused_norm_and_silu", 1), ("eager_grouped_gemv", 2),
                         ("eager_grouped_gemv_fused_attention", 3), ("eager_split_norms", 4),
                         ("eager_qkv_and_attention_in_one_launch", 5)):
-        dec.time_steps(tok, n_past, fused, 3)
+        dec.time_steps(tok, n_past, fused, SETTLE_STEPS)
         ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
         res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
         plan_logits[fused] = dec.logits().astype(np.float64)
@@ -248,7 +274,7 @@ def decode_step_bench(dev, reps, with_graph=True):
     graph_logits = {}
     for name, fused in (("hip_graph_split_norms", 4), ("hip_graph_qkv_and_attention_in_one_launch", 5)):
         dec.capture(tok, n_past, fused)
-        dec.time_replays(3)
+        dec.time_replays(SETTLE_STEPS)
         ms = min(dec.time_replays(reps) for _ in range(3)) / reps
         res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
                      "GBps": round((weight_bytes + kv_bytes) / ms / 1e6, 1),
@@ -270,7 +296,7 @@ def decode_step_bench(dev, reps, with_graph=True):
     # contents: the logits are compared with the one-kernel-per-op plan of the [n_ctx][n_embd] decoder above)
     dec, _ = make_decoder(False, True)
     for name, fused in (("eager_split_norms_head_major_kv", 4), ("eager_qkv_and_attention_in_one_launch_head_major_kv", 5)):
-        dec.time_steps(tok, n_past, fused, 3)
+        dec.time_steps(tok, n_past, fused, SETTLE_STEPS)
         ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
         res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
                      "GBps": round((weight_bytes + kv_bytes) / ms / 1e6, 1),
@@ -281,7 +307,7 @@ def decode_step_bench(dev, reps, with_graph=True):
     dec, _ = make_decoder(True)
     b16 = weight_bytes + kv_bytes // 2
     for name, fused in (("eager_split_norms_f16_kv", 4), ("eager_qkv_and_attention_in_one_launch_f16_kv", 5)):
-        dec.time_steps(tok, n_past, fused, 3)
+        dec.time_steps(tok, n_past, fused, SETTLE_STEPS)
         ms = min(dec.time_steps(tok, n_past, fused, reps) for _ in range(3)) / reps
         res[name] = {
             "launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1),
@@ -370,8 +396,8 @@ def main():
         f = lambda i, j=j, k=k, n=n: dev.dequantize_mul_mat_vec_q4_0(sets[i % nsets][j], xs[k], ys[j], k, n)
         for i in range(20):
             f(i)
-        us = timed(dev, f, 200, reps=5) / 200 * 1e3
-        us_graph = timed_graph(dev, f, 200) / 200 * 1e3   # the same launches replayed from a HIP graph: no host in the loop
+        us = timed(dev, f, 200, reps=5, settle_s=SETTLE_S) / 200 * 1e3
+        us_graph = timed_graph(dev, f, 200, settle_s=SETTLE_S) / 200 * 1e3   # the same launches replayed from a HIP graph: no host in the loop
         per_shape.append({"K": k, "N": n, "us": round(us, 3), "us_graph_replay": round(us_graph, 3),
                           "weight_GBps": round(q4_bytes(k, n) / us / 1e3, 1),
                           "hbm_frac": round(q4_bytes(k, n) / us / 1e3 / HBM_PEAK_GBPS, 4)})
@@ -388,7 +414,7 @@ def main():
         wp = base[1]  # K=4096 -> N=11008
         for _ in range(50):  # warm: the fp16 workspace is allocated on the first call, clocks settle
             dev.mul_mat_q4_0_f32(wp, xp, yp, k, n, m)
-        us = timed(dev, lambda i: dev.mul_mat_q4_0_f32(wp, xp, yp, k, n, m), 100, reps=5) / 100 * 1e3
+        us = timed(dev, lambda i: dev.mul_mat_q4_0_f32(wp, xp, yp, k, n, m), 100, reps=5, settle_s=SETTLE_S) / 100 * 1e3
         tf = 2.0 * m * k * n / us / 1e6
         extra["prefill_gemm"] = {"M": m, "K": k, "N": n, "us": round(us, 2), "TFLOPs": round(tf, 1),
                                  "roofline": {"bound": "mfma", "achieved": round(tf, 1),
@@ -401,11 +427,47 @@ def main():
             yo = dev.alloc(m * n2 * 4)
             for _ in range(20):
                 dev.mul_mat_q4_0_f32(wq, xo, yo, k2, n2, m)
-            uso = timed(dev, lambda i: dev.mul_mat_q4_0_f32(wq, xo, yo, k2, n2, m), 50, reps=5) / 50 * 1e3
+            uso = timed(dev, lambda i: dev.mul_mat_q4_0_f32(wq, xo, yo, k2, n2, m), 50, reps=5, settle_s=SETTLE_S) / 50 * 1e3
             others.append({"M": m, "K": k2, "N": n2, "us": round(uso, 2), "TFLOPs": round(2.0 * m * k2 * n2 / uso / 1e6, 1)})
             dev.free(xo)
             dev.free(yo)
         extra["prefill_gemm_other_shapes"] = others
+        # The same matmul on activations that are already an fp16 panel (written once by the op that produces them:
+        # a conversion, an RMSNorm or a SwiGLU), and several matrices of a layer against one panel in one launch.  These
+        # are NOT the configs[2] figure above (there X is f32 and is converted inside the timed call); they are what a
+        # prefill graph built on the panel calls sees.
+        pb = dev.alloc(dev.f16_panel_bytes(k, m))
+        dev.f32_to_f16_panel(xp, pb, k, m)
+        gnorm = dev.upload((1 + 0.1 * rng.standard_normal(k)).astype(np.float32))
+        w3 = [base[0]] + [dev.alloc(q4_bytes(4096, 4096)) for _ in range(2)]
+        for c in w3[1:]:
+            dev.copy_d2d(c, base[0], q4_bytes(4096, 4096))
+        w2 = [wp, sets[1][1]]
+        y3 = [dev.alloc(m * 4096 * 4) for _ in range(3)]
+        y2 = [yp, dev.alloc(m * n * 4)]
+        panel = {}
+
+        def tpanel(name, fn, flop, calls=50):
+            for _ in range(20):
+                fn()
+            usp = timed(dev, lambda i: fn(), calls, reps=5, settle_s=SETTLE_S) / calls * 1e3
+            panel[name] = {"us": round(usp, 2)}
+            if flop:
+                panel[name].update(TFLOPs=round(flop / usp / 1e6, 1), mfma_frac=round(flop / usp / 1e6 / MFMA_F16_PEAK_TFLOPS, 4))
+
+        tpanel("f32_to_panel_512x4096", lambda: dev.f32_to_f16_panel(xp, pb, k, m), 0)
+        tpanel("rms_norm_mul_to_panel_512x4096", lambda: dev.rms_norm_mul_f16_panel(xp, gnorm, pb, k, m, 1e-6), 0)
+        dev.f32_to_f16_panel(xp, pb, k, m)
+        tpanel("matmul_512x4096x11008", lambda: dev.mul_mat_q4_0_f16_panel([(wp, yp, n)], pb, k, m), 2.0 * m * k * n)
+        tpanel("gate_up_one_launch_512x4096x2x11008",
+               lambda: dev.mul_mat_q4_0_f16_panel([(w, y, n) for w, y in zip(w2, y2)], pb, k, m), 2 * 2.0 * m * k * n)
+        tpanel("qkv_one_launch_512x4096x3x4096",
+               lambda: dev.mul_mat_q4_0_f16_panel([(w, y, 4096) for w, y in zip(w3, y3)], pb, k, m), 3 * 2.0 * m * k * 4096)
+        tpanel("qkv_three_f32_calls_512x4096x4096",
+               lambda: [dev.mul_mat_q4_0_f32(w, xp, y, k, 4096, m) for w, y in zip(w3, y3)], 3 * 2.0 * m * k * 4096)
+        extra["prefill_gemm_fp16_panel"] = panel
+        for b_ in [pb, gnorm, y2[1]] + w3[1:] + y3:
+            dev.free(b_)
         # row kernels (configs[3]); algorithmic bytes: rms_norm + weight = read + write of 512 x 4096 f32 + the weight
         # row, rope = read + write + positions, causal softmax = lower triangle read + full write of 32 x 512 x 512 f32
         # Inputs and outputs rotate over enough copies (> 256 MB in total) that no launch finds its rows in the
@@ -418,13 +480,13 @@ def main():
         outs = [dev.alloc(512 * 4096 * 4) for _ in range(nrot)]
         g = dev.upload((1 + 0.1 * rng.standard_normal(4096)).astype(np.float32))
         f = lambda i: dev.rms_norm_mul_f32(ins[i % nrot], g, outs[i % nrot], 4096, 512, 1e-6)
-        us = timed_graph(dev, f, 100) / 100 * 1e3
+        us = timed_graph(dev, f, 100, settle_s=SETTLE_S) / 100 * 1e3
         rows["rms_norm_mul"] = {"us": round(us, 3), "GBps": round(16793600 / us / 1e3, 1),
                                 "us_eager": round(timed(dev, f, 100, reps=5) / 100 * 1e3, 3)}
         pos = dev.upload(np.arange(512, dtype=np.int32))
         ts = float(np.float32(10000.0) ** np.float32(-2.0 / 128))
         f = lambda i: dev.rope_f32(ins[i % nrot], outs[i % nrot], 128, 512 * 32, pos, 1.0, 32, ts)
-        us = timed_graph(dev, f, 100) / 100 * 1e3
+        us = timed_graph(dev, f, 100, settle_s=SETTLE_S) / 100 * 1e3
         rows["rope"] = {"us": round(us, 3), "GBps": round(16779264 / us / 1e3, 1),
                         "us_eager": round(timed(dev, f, 100, reps=5) / 100 * 1e3, 3)}
         for b_ in ins + outs:
@@ -434,7 +496,7 @@ def main():
         sin = [dev.upload(s_host) for _ in range(nrot)]
         sout = [dev.alloc(32 * 512 * 512 * 4) for _ in range(nrot)]
         f = lambda i: dev.soft_max_causal_f32(sin[i % nrot], sout[i % nrot], 512, 512, 32 * 512, 0)
-        us = timed_graph(dev, f, 100) / 100 * 1e3
+        us = timed_graph(dev, f, 100, settle_s=SETTLE_S) / 100 * 1e3
         rows["soft_max_causal"] = {"us": round(us, 3), "GBps": round(50364416 / us / 1e3, 1),
                                    "us_eager": round(timed(dev, f, 100, reps=5) / 100 * 1e3, 3)}
         for b_ in sin + sout:
