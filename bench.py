@@ -38,8 +38,8 @@ PREFILL = (512, 4096, 11008)    # (M, K, N)
 ROTATE_BYTES = 1200 << 20
 # HBM bytes per grouped launch (the four products) measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE on
 # this workload, each scaled by what the same counter reads for a device-to-device copy of known size
-# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); see profiles/gemv_q4_0_group__llama7b_gemv_set.md
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 135240090
+# (FETCH_SIZE x 1.9992, WRITE_SIZE x 1.000); see profiles/gemv_q4_0_group__llama7b_gemv_set.md
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 135187713
 
 
 def q4_bytes(k, n):
@@ -99,9 +99,15 @@ def timed(dev, fn, iters, reps=1, settle_s=0.0):
     return float(np.median(out))
 
 
+USE_GRAPHS = True   # --no-graph: every graph-replay measurement falls back to eager launches (rocprofv3's kernel
+                    # tracer does not survive thousands of graph launches)
+
+
 def timed_graph(dev, fn, iters, reps=5, settle_s=0.0):
     """As timed(), with the `iters` launches recorded once into a HIP graph and replayed: the figure for kernels
     short enough that issuing them one by one from Python is what an eager loop measures."""
+    if not USE_GRAPHS:
+        return timed(dev, fn, iters, reps, settle_s)
     dev.synchronize()
     dev.graph_begin_capture()
     for i in range(iters):
@@ -329,7 +335,14 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode-step measurement")
     ap.add_argument("--decode-no-graph", action="store_true",
                     help="decode step: eager launches only (graph replays cannot run under the kernel tracer)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="no HIP-graph replays anywhere: graph figures are measured as eager launches (for runs under "
+                         "rocprofv3 --kernel-trace); implies --decode-no-graph")
     args = ap.parse_args()
+    global USE_GRAPHS
+    if args.no_graph:
+        USE_GRAPHS = False
+        args.decode_no_graph = True
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on ONE GPU (no collectives, no sharding); "
                          "--gpus %d is not supported, run with --gpus 1\n" % args.gpus)
