@@ -206,6 +206,39 @@ def _normal_f32(seed, count, scale, threads=16):
     return out
 
 
+def decode_attention_bench(dev, rng):
+    """The decode step's attention launches alone (BASELINE configs[4]'s shapes: 32 heads of 128, KV length 2048, f32
+    caches): galois_hip_attn_decode_f32, and galois_hip_qkv_attn_decode_f32 with its three 4096 x 4096 products, over
+    six copies of the caches in rotation (805 MB: no launch finds its rows in the Infinity Cache)."""
+    H, D, L = 32, 128, 2048
+    E = H * D
+    nbuf = 6
+    kcs = [dev.upload(rng.standard_normal((L, E), dtype=np.float32)) for _ in range(nbuf)]
+    vcs = [dev.alloc(L * E * 4) for _ in range(nbuf)]
+    for v_, k_ in zip(vcs, kcs[::-1]):
+        dev.copy_d2d(v_, k_, L * E * 4)
+    q, k, v = (dev.upload(rng.standard_normal(E, dtype=np.float32)) for _ in range(3))
+    out = dev.alloc(E * 4)
+    pos = dev.upload(np.array([L - 1], np.int32))
+    ws = [make_q4_matrix(dev, rng, E, E) for _ in range(3)]
+    x = dev.upload(rng.standard_normal(E, dtype=np.float32))
+    items = dev.gemv_items([{"vx": w, "y": x, "dst": d, "ncols": E, "nrows": E} for w, d in zip(ws, (q, k, v))])
+    ts = float(np.float32(10000.0) ** np.float32(-2.0 / D))
+    cache_bytes = 2 * L * E * 4
+    res = {}
+    for name, f, nbytes in (
+            ("attn_decode_f32", lambda i: dev.attn_decode_f32(q, k, v, kcs[i % nbuf], vcs[i % nbuf], out, H, D, L - 1, pos,
+                                                              1.0, ts, D ** -0.5), cache_bytes),
+            ("qkv_attn_decode_f32", lambda i: dev.qkv_attn_decode(items, kcs[i % nbuf], vcs[i % nbuf], out, H, D, L - 1,
+                                                                   pos, 1.0, ts, D ** -0.5), cache_bytes + 3 * q4_bytes(E, E))):
+        us = timed_graph(dev, f, 60, settle_s=SETTLE_S) / 60 * 1e3
+        res[name] = {"us": round(us, 3), "algorithmic_bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                     "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    for b_ in kcs + vcs + ws + [q, k, v, out, pos, x]:
+        dev.free(b_)
+    return res
+
+
 SETTLE_STEPS = 150   # decode steps (1.6-3 ms each) run before a plan is timed: the same settling as SETTLE_S
 
 
@@ -517,6 +550,7 @@ def main():
         for v in rows.values():
             v["hbm_frac"] = round(v["GBps"] / HBM_PEAK_GBPS, 4)
         extra["row_kernels"] = rows
+        extra["decode_attention"] = decode_attention_bench(dev, rng)
 
     out = {
         "metric": "Q4_0 GEMV weight GB/s (% of HBM peak); Q4_0 prefill GEMM TFLOP/s @7B shapes",
