@@ -300,6 +300,27 @@ def decode_step_bench(dev, reps, with_graph=True):
         return {"max_rel": float(np.max(np.abs(a - b)) / np.max(np.abs(b))),
                 "l2_rel": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
 
+    def prefill(dec, n_tok=512):
+        """n_tok tokens from an empty context in one pass (LlamaDecoder.prefill: the Q4_0 products through the prefill
+        matmul on fp16 panels) against the same tokens decoded one by one on the same decoder."""
+        hp = dec.hp
+        e, f = hp["n_embd"], hp["n_ff"]
+        toks = np.random.default_rng(11).integers(0, hp["n_vocab"], n_tok).astype(np.int32)
+        for i, t in enumerate(toks):
+            dec.decode(int(t), i, 5)
+        one_by_one = dec.logits().astype(np.float64)
+        dec.prefill(toks, 0)
+        got = dec.logits().astype(np.float64)
+        dec.time_prefill(toks, 0, 4)
+        ms = min(dec.time_prefill(toks, 0, 4) for _ in range(3)) / 4
+        q4_flop = 2.0 * n_tok * hp["n_layer"] * (4 * e * e + 3 * e * f)
+        attn_flop = 2.0 * 2 * n_tok * n_tok * e * hp["n_layer"]     # scores and out over all n_tok keys (the masked half too)
+        return {"tokens": n_tok, "launches": dec.ops_per_prefill(), "ms": round(ms, 3), "tokens_per_s": round(n_tok / ms * 1e3, 0),
+                "q4_0_products_TFLOPs_if_alone": round(q4_flop / ms / 1e9, 1),
+                "q4_0_flop": q4_flop, "attention_flop": attn_flop,
+                "speedup_over_decoding_one_by_one": round(n_tok * res["eager_qkv_and_attention_in_one_launch"]["ms_per_token"] / ms, 1),
+                "last_logits_vs_one_by_one": cross(got, one_by_one)}
+
     for name, fused in (("eager_one_kernel_per_op", 0), ("eager_fused_norm_and_silu", 1), ("eager_grouped_gemv", 2),
                         ("eager_grouped_gemv_fused_attention", 3), ("eager_split_norms", 4),
                         ("eager_qkv_and_attention_in_one_launch", 5)):
@@ -308,6 +329,7 @@ def decode_step_bench(dev, reps, with_graph=True):
         res[name] = {"launches": dec.ops_per_step(), "ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
         plan_logits[fused] = dec.logits().astype(np.float64)
     if not with_graph:
+        res["prefill_512_tokens"] = prefill(dec)
         dec.close()
         return res
     graph_logits = {}
@@ -330,6 +352,7 @@ def decode_step_bench(dev, reps, with_graph=True):
         **{k: cross(v, plan_logits[0]) for k, v in graph_logits.items()}}
     res["logits_within_1e-4"] = bool(all(v["max_rel"] < 1e-4 and v["l2_rel"] < 1e-4
                                          for v in res["logits_vs_one_kernel_per_op"].values()))
+    res["prefill_512_tokens"] = prefill(dec)
     dec.close()
     # the same step with the caches kept [n_head][n_ctx][head_dim]: a head's keys contiguous (same weights, same cache
     # contents: the logits are compared with the one-kernel-per-op plan of the [n_ctx][n_embd] decoder above)
@@ -353,6 +376,7 @@ def decode_step_bench(dev, reps, with_graph=True):
             "algorithmic_bytes_per_token": b16, "GBps": round(b16 / ms / 1e6, 1),
             "hbm_frac": round(b16 / ms / 1e6 / HBM_PEAK_GBPS, 4),
             "logits_finite": bool(np.all(np.isfinite(dec.logits())))}
+    res["prefill_512_tokens_f16_kv"] = prefill(dec)
     dec.close()
     return res
 

@@ -280,6 +280,13 @@ class Device:
         self._check(fn(self._ctx, arr, _ptr(k_cache), _ptr(v_cache), _ptr(out), n_head, head_dim, n_past, _ptr(pos),
                        freq_scale, theta_scale, scale, head_major_n_ctx))
 
+    def attn_prefill(self, q, k_cache, v_cache, out, out_panel, n_head, head_dim, n_tokens, n_past, scale, kv_f16=False):
+        """Causal attention of n_tokens rows of q over caches that already hold positions 0 .. n_past + n_tokens - 1;
+        the result goes to out (f32) or out_panel (fp16 panel), the other is None."""
+        fn = self._lib.galois_hip_attn_prefill_f16kv if kv_f16 else self._lib.galois_hip_attn_prefill_f32
+        self._check(fn(self._ctx, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out) if out is not None else None,
+                       _ptr(out_panel) if out_panel is not None else None, n_head, head_dim, n_tokens, n_past, scale))
+
     def attn_decode_f16kv(self, q, k, v, k_cache, v_cache, out, n_head, head_dim, n_past, pos, freq_scale, theta_scale,
                           scale, head_major_n_ctx=0):
         self._check(self._lib.galois_hip_attn_decode_f16kv(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache),

@@ -78,6 +78,8 @@ PROTOTYPES = {
     "galois_hip_attn_decode_f32_static": (i32, [c_ctx, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, f32, f32, f32, i32]),
     "galois_hip_attn_decode_f16kv": (i32, [c_ctx, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, f32, f32, f32, i32]),
     "galois_hip_qkv_attn_decode_f32": (i32, [c_ctx, C.POINTER(GemvItem), vp, vp, vp, i32, i32, i32, vp, f32, f32, f32, i32]),
+    "galois_hip_attn_prefill_f32": (i32, [c_ctx, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]),
+    "galois_hip_attn_prefill_f16kv": (i32, [c_ctx, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]),
     "galois_hip_qkv_attn_decode_f16kv": (i32, [c_ctx, C.POINTER(GemvItem), vp, vp, vp, i32, i32, i32, vp, f32, f32, f32, i32]),
     "galois_hip_mul_mat_f16_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32, i32, i32, C.c_int64, C.c_int64, C.c_int64]),
     "galois_hip_mul_mat_f32": (i32, [c_ctx, vp, vp, vp, i32, i32, i32, i32, i32, C.c_int64, C.c_int64, C.c_int64]),

@@ -190,6 +190,28 @@ int galois_host_llama_decode(void *m, int32_t token, int32_t n_past, int fused) 
     GResult r = ((LlamaDecoder *)m)->decode(token, n_past, fused);
     return r.ok() ? 0 : fail(r);
 }
+int galois_host_llama_prefill(void *m, const int32_t *tokens, size_t n, int32_t n_past) {
+    GResult r = ((LlamaDecoder *)m)->prefill(tokens, n, n_past);
+    return r.ok() ? 0 : fail(r);
+}
+size_t galois_host_llama_ops_per_prefill(void *m) { return ((LlamaDecoder *)m)->ops_per_prefill(); }
+// `reps` prefills of the same tokens between two events; milliseconds for all of them in *ms
+int galois_host_llama_time_prefill(void *m, void *dev, const int32_t *tokens, size_t n, int32_t n_past, int reps, float *ms) {
+    galois_hip_ctx *ctx = ((Device *)dev)->gpu->ctx();
+    galois_hip_event *e0 = nullptr, *e1 = nullptr;
+    int32_t st = galois_hip_event_create(ctx, &e0);
+    if (!st) st = galois_hip_event_create(ctx, &e1);
+    if (!st) st = galois_hip_event_record(ctx, e0);
+    GResult r;
+    for (int i = 0; i < reps && !st && r.ok(); i++) r = ((LlamaDecoder *)m)->prefill(tokens, n, n_past);
+    if (!st) st = galois_hip_event_record(ctx, e1);
+    if (!st) st = galois_hip_event_elapsed_ms(ctx, e0, e1, ms);
+    galois_hip_event_destroy(ctx, e0);
+    galois_hip_event_destroy(ctx, e1);
+    if (!r.ok()) return fail(r);
+    if (st) return fail(((Device *)dev)->gpu->check(st));
+    return 0;
+}
 int galois_host_llama_capture(void *m, int32_t token, int32_t n_past, int fused) {
     GResult r = ((LlamaDecoder *)m)->capture(token, n_past, fused);
     return r.ok() ? 0 : fail(r);

@@ -50,6 +50,16 @@ class LlamaDecoder {
     // Records the same step as a graph / replays the recorded step.
     GResult capture(int32_t token, int32_t n_past, int fused);
     GResult replay();
+    // Prefill: `n` tokens at positions n_past .. n_past + n - 1 in one pass (llama_prefill.cpp).  The same graph as n
+    // decode steps, issued with the many-row ops: the Q4_0 products through the prefill matmul on fp16 panels that the
+    // norms and the SwiGLU write directly (q | k | v and gate | up one launch each), rope_custom over all positions,
+    // the n new rows of both caches appended at once, scores = K^T Q and out = V P per head on the matrix cores with
+    // a causal soft_max between them (heads of 128: galois_attn_prefill instead, one launch that writes the panel of
+    // the output projection; f32 caches then also receive the rotated keys and the values directly).  Afterwards the caches hold positions 0 .. n_past + n - 1 and logits() the last
+    // token's.  n_embd and n_ff must be multiples of 256; caches [n_embd, n_ctx] (not head-major), f32 or f16.
+    // Intermediates are sized for the largest n and n_past + n seen so far (this call allocates when they grow).
+    GResult prefill(const int32_t *tokens, size_t n, int32_t n_past);
+    size_t ops_per_prefill() const { return n_prefill_ops_; }
     const Tensor &logits() const { return logits_; }
     const LlamaHParams &hparams() const { return hp_; }
     size_t ops_per_step() const { return n_ops_; }
@@ -68,8 +78,14 @@ class LlamaDecoder {
     Tensor tok_id_, pos_, scale_;                                    // I32 [1], I32 [1], host f32 [1]
     Tensor x_, t_, a_, q_, k_, v_, qr_, kr_, s_, p_, o_, ao_, x1_, f_, g_, u_, h_, d_, logits_;
     Tensor ssq_, ssq1_;  // partial sums of squares of x and x1 (fused = 4)
+    struct Prefill {  // intermediates of prefill(), for up to `rows` tokens attending over up to `keys` positions
+        size_t rows = 0, keys = 0;
+        Tensor tok, pos, x, x1, t, q, k, v, qr, kr, q3, s, p, o, ao, g, u, panel_e, panel_f;
+    };
+    GResult prefill_buffers(size_t n, size_t keys);
+    Prefill pf_;
     galois_hip_graph *graph_ = nullptr;
-    size_t n_ops_ = 0;
+    size_t n_ops_ = 0, n_prefill_ops_ = 0;
     int32_t last_token_ = -1, last_pos_ = -1;
 };
 
@@ -93,11 +109,30 @@ struct MatvecItem {
 };
 GResult galois_matvec_group(const std::vector<MatvecItem> &items);
 
+// The prefill matmul's fp16 panel (galois_hip_*_f16_panel): `panel` is an F16 tensor of galois_panel_elems(K, M)
+// elements.  The producers write rms_norm(src, eps) * weight, silu(gate) * up, or src itself, for src = [K, M] f32;
+// galois_matmul_panel multiplies one to four Q4_0 matrices [K, N_j] by it in one launch, dst_j = [N_j, M] f32.
+size_t galois_panel_elems(size_t K, size_t M);
+GResult galois_rms_norm_mul_panel(const Tensor &src, const Tensor &weight, Tensor &panel, float eps);
+GResult galois_silu_mul_panel(const Tensor &gate, const Tensor &up, Tensor &panel);
+GResult galois_to_panel(const Tensor &src, Tensor &panel);
+struct PanelMatmulItem {
+    const Tensor *w = nullptr;
+    Tensor *dst = nullptr;
+};
+GResult galois_matmul_panel(const std::vector<PanelMatmulItem> &items, const Tensor &panel, size_t K, size_t M);
+
 // Attention of one decode step in one launch (galois_hip_attn_decode_f32): rope_custom of q and k at position
 // pos[0] = n_past, append of k and v to row n_past of the caches ([n_embd, n_ctx], both f32 or both f16), scores = K^T q scaled
 // by `scale`, soft_max over the n_past + 1 keys and out = V p, for n_head heads of q.dim / n_head elements.
 GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                            Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale);
+
+// Causal attention of all rows of q ([n_embd, n] f32, rotated) over caches ([n_embd, n_ctx], both f32 or both f16) that
+// already hold positions 0 .. n_past + n - 1, in one launch (galois_hip_attn_prefill_f32 / _f16kv; heads of 128).
+// dst is either an F32 tensor [n_embd, n] or an F16 panel of galois_panel_elems(n_embd, n) elements.
+GResult galois_attn_prefill(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &dst, size_t n_head,
+                            int32_t n_past, float scale);
 
 // The three products q | k | v (as galois_matvec_group takes them; plain or normalising) and the attention that
 // consumes them (galois_attn_decode on their dst tensors) in one launch (galois_hip_qkv_attn_decode_f32 / _f16kv).

@@ -61,6 +61,10 @@ def lib():
                 ("galois_host_llama_free", None, [vp]), ("galois_host_llama_tensor", vp, [vp, C.c_char_p, C.c_int]),
                 ("galois_host_llama_logits", vp, [vp]), ("galois_host_llama_ops_per_step", sz, [vp]),
                 ("galois_host_llama_decode", C.c_int, [vp, C.c_int32, C.c_int32, C.c_int]),
+                ("galois_host_llama_prefill", C.c_int, [vp, C.POINTER(C.c_int32), sz, C.c_int32]),
+                ("galois_host_llama_ops_per_prefill", sz, [vp]),
+                ("galois_host_llama_time_prefill", C.c_int, [vp, vp, C.POINTER(C.c_int32), sz, C.c_int32, C.c_int,
+                                                             C.POINTER(C.c_float)]),
                 ("galois_host_llama_capture", C.c_int, [vp, C.c_int32, C.c_int32, C.c_int]),
                 ("galois_host_llama_replay", C.c_int, [vp]),
                 ("galois_host_llama_time_replays", C.c_int, [vp, vp, C.c_int, C.POINTER(C.c_float)]),
@@ -278,6 +282,21 @@ class LlamaDecoder:
 
     def decode(self, token, n_past, fused=False):
         _call(lib().galois_host_llama_decode(self.h, token, n_past, int(fused)))
+
+    def prefill(self, tokens, n_past=0):
+        """All of `tokens` at positions n_past .. in one pass; afterwards the caches hold them and logits() the last one's."""
+        t = np.ascontiguousarray(tokens, np.int32)
+        _call(lib().galois_host_llama_prefill(self.h, t.ctypes.data_as(C.POINTER(C.c_int32)), t.size, n_past))
+
+    def ops_per_prefill(self):
+        return lib().galois_host_llama_ops_per_prefill(self.h)
+
+    def time_prefill(self, tokens, n_past, reps):
+        t = np.ascontiguousarray(tokens, np.int32)
+        ms = C.c_float()
+        _call(lib().galois_host_llama_time_prefill(self.h, self.device.h, t.ctypes.data_as(C.POINTER(C.c_int32)), t.size, n_past,
+                                                   reps, C.byref(ms)))
+        return ms.value
 
     def capture(self, token, n_past, fused=False):
         _call(lib().galois_host_llama_capture(self.h, token, n_past, int(fused)))

@@ -357,6 +357,30 @@ int32_t galois_hip_qkv_attn_decode_f16kv(galois_hip_ctx *ctx, const galois_hip_g
                                          void *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
                                          const int32_t *pos, float freq_scale, float theta_scale, float scale, int32_t head_major_n_ctx);
 
+/* Causal attention of n_tokens query rows over a KV cache in ONE launch: what a prefill issues per layer as
+ * cpy(q -> [D, M, H]), matmul(K^T, q), scale, soft_max under the causal mask, matmul(V, p), cpy(-> [D, H, M])
+ * (CudaMatMul src/cuda.rs:867-992, scale and soft_max src/cuda.rs:1597-1663 and 1257-1356, cpy src/cuda.rs:1382-1595),
+ * without the scores ever reaching memory:
+ *   q: [n_tokens][n_head * head_dim] f32, rotated; k_cache, v_cache: [>= n_past + n_tokens][n_head * head_dim] rows that
+ *   already hold positions 0 .. n_past + n_tokens - 1 (this call appends nothing);
+ *   row m of head h of the result = sum_l softmax_l(scale * q[m]_h . K[l]_h) V[l]_h over l = 0 .. n_past + m.
+ * The result goes to out ([n_tokens][n_head * head_dim] f32) or to out_panel (the fp16 panel of that [n_head * head_dim,
+ * n_tokens] operand, galois_hip_f16_panel_bytes(n_head * head_dim, n_tokens) bytes, ready for
+ * galois_hip_mul_mat_q4_0_f16_panel): exactly one of the two is non-null.
+ * Arithmetic: both products run on the matrix cores with fp16 operands and f32 sums, as the reference's gemm_ex on
+ * converted operands does (convert_fp32_to_fp16, src/cuda.rs:881-992): q * scale * log2(e), the keys, the values and
+ * the probabilities are rounded to fp16 (an f16 cache is read as it is), maxima, sums and the output accumulate in f32.
+ * Against f64 arithmetic on the same inputs the result is within 2e-3 of the largest output magnitude for scores of a
+ * few units (unit-variance q and k); rounding q and k moves a score by about 2^-11 of the size of its terms and the
+ * exponential makes that a relative error of the probabilities, so scores of +-100 are held to 5e-3.
+ * head_dim 128; all pointers 16-byte aligned. */
+int32_t galois_hip_attn_prefill_f32(galois_hip_ctx *ctx, const float *q, const float *k_cache, const float *v_cache, float *out,
+                                    void *out_panel, int32_t n_head, int32_t head_dim, int32_t n_tokens, int32_t n_past,
+                                    float scale);
+int32_t galois_hip_attn_prefill_f16kv(galois_hip_ctx *ctx, const float *q, const void *k_cache, const void *v_cache, float *out,
+                                      void *out_panel, int32_t n_head, int32_t head_dim, int32_t n_tokens, int32_t n_past,
+                                      float scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -360,3 +360,84 @@ def test_32_layers_at_kv_length_2048_against_the_oracle(gdev):
     for plan, (emax, el2) in worst.items():
         assert emax < 2e-4 and el2 < 2e-4, (plan, emax, el2)
         assert emax < 2 * f32_max and el2 < 2 * f32_l2, (plan, emax, el2, f32_max, f32_l2)
+
+
+def _ref_tokens(w, hp, kc, vc, tokens, n_past, round_kv=False):
+    """The oracle's step for each of `tokens` in turn from position n_past; the last token's logits."""
+    for i, tok in enumerate(tokens):
+        ref = _ref_step(w, hp, kc, vc, int(tok), n_past + i, round_kv)
+    return ref
+
+
+# The prefill products take their activations rounded to f16 (the Q4_0 prefill matmul and, for several rows, the f16
+# matmul of an f16 cache): 2^-11 relative per element, against the decode step's exact f32 activations.
+PREFILL_TOL = 3e-3
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+@pytest.mark.parametrize("n_head", [2, 4])
+def test_prefill_matches_the_oracle_token_by_token(gdev, kv_f16, n_head):
+    """Two prefill calls (an empty cache, then a filled one; 20 and 9 tokens: neither a multiple of the panel's 16
+    rows) and a decode step on the caches they left, each against the oracle's one-token step run over the same tokens.
+    Heads of 128 (n_head = 2) take the attention as one launch, heads of 64 as the op sequence."""
+    rng = np.random.default_rng(57)
+    hp = dict(SMALL, n_head=n_head)
+    w = _make_weights(rng, hp)
+    dec = g.LlamaDecoder(gdev, kv_f16=kv_f16, **hp)
+    _load(dec, w)
+    kc = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float32)
+    vc = np.zeros_like(kc)
+    toks = rng.integers(0, hp["n_vocab"], 30).astype(np.int32)
+    ref = _ref_tokens(w, hp, kc, vc, toks[:20], 0, kv_f16)
+    dec.prefill(toks[:20], 0)
+    _check(dec.logits(), ref, PREFILL_TOL)
+    # launches: embedding lookup, per layer 20 (f16 caches: two copies into them) or 18 with the op-sequence attention
+    # and 14 or 12 with the attention in one launch, then the last row's copy, norm and lm head
+    per_layer = (12 if n_head == 2 else 18) + (2 if kv_f16 else 0)
+    assert dec.ops_per_prefill() == 1 + hp["n_layer"] * per_layer + 3
+    ref = _ref_tokens(w, hp, kc, vc, toks[20:29], 20, kv_f16)
+    dec.prefill(toks[20:29], 20)
+    _check(dec.logits(), ref, PREFILL_TOL)
+    for i in range(hp["n_layer"]):
+        kg = dec.tensor("k_cache", i).to_cpu_tensor().astype(np.float32)
+        vg = dec.tensor("v_cache", i).to_cpu_tensor().astype(np.float32)
+        assert not kg[29:].any() and not vg[29:].any()
+        _check(kg[:29], kc[i][:29], PREFILL_TOL)
+        _check(vg[:29], vc[i][:29], PREFILL_TOL)
+    ref = _ref_step(w, hp, kc, vc, int(toks[29]), 29, kv_f16)
+    dec.decode(int(toks[29]), 29, 5 if n_head == 2 else 4)
+    _check(dec.logits(), ref, PREFILL_TOL)
+    dec.close()
+
+
+def test_prefill_of_one_token_and_its_refusals(gdev):
+    rng = np.random.default_rng(58)
+    hp = SMALL
+    w = _make_weights(rng, hp)
+    dec = g.LlamaDecoder(gdev, **hp)
+    _load(dec, w)
+    kc = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float32)
+    vc = np.zeros_like(kc)
+    ref = _ref_step(w, hp, kc, vc, 7, 0)
+    dec.prefill([7], 0)
+    _check(dec.logits(), ref, PREFILL_TOL)
+    # a full context in one call
+    toks = rng.integers(0, hp["n_vocab"], hp["n_ctx"] - 1).astype(np.int32)
+    ref = _ref_tokens(w, hp, kc, vc, toks, 1)
+    dec.prefill(toks, 1)
+    _check(dec.logits(), ref, PREFILL_TOL)
+    for bad in (([], 0), ([1, 2], hp["n_ctx"] - 1), ([1], -1), ([hp["n_vocab"]], 0)):
+        with pytest.raises(g.GError) as e:
+            dec.prefill(*bad)
+        assert e.value.kind == "ShapeError"
+    dec.close()
+    hm = g.LlamaDecoder(gdev, kv_head_major=True, **hp)
+    with pytest.raises(g.GError) as e:
+        hm.prefill([1, 2, 3], 0)
+    assert e.value.kind == "Unimplemented"
+    hm.close()
+    narrow = g.LlamaDecoder(gdev, **dict(hp, n_embd=128, n_head=1))
+    with pytest.raises(g.GError) as e:
+        narrow.prefill([1, 2, 3], 0)
+    assert e.value.kind == "Unimplemented"
+    narrow.close()
