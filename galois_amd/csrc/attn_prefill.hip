@@ -36,12 +36,14 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr int PA_D = 128;                  // head dim
 constexpr int PA_BK = 32;                  // keys per block
-constexpr int PA_THREADS = 256;
+constexpr int PA_THREADS = 512;
 constexpr int PA_KROW = 272;               // bytes per key row of the K tile (256 + 16: fragment reads hit every bank once)
 constexpr int PA_VROW = 80;                // bytes per dim row of the transposed V tile (32 slots of fp16 + 16)
 constexpr int PA_KBYTES = PA_BK * PA_KROW;  // 8704
 constexpr int PA_VBYTES = PA_D * PA_VROW;   // 10240
-constexpr int PA_STAGE = PA_KBYTES + PA_VBYTES;
+constexpr int PA_BLOCK = PA_KBYTES + PA_VBYTES;  // one block of 32 keys in LDS
+constexpr int PA_STAGE = 2 * PA_BLOCK;            // a stage: two blocks, one per half of the workgroup
+constexpr int PA_LDS = 2 * PA_STAGE;              // 75,776 bytes
 
 struct pa_args {
     const float *q;     // [n][n_head * 128], rotated
@@ -68,50 +70,78 @@ __device__ __forceinline__ uint4 pa_pack8(const float4 a, const float4 b) {
 // group's index, so that the sixteen threads that store the same element of their eight dims hit different banks.
 __device__ __forceinline__ int pa_vrow(int d) { return (d & ~7) | ((d + (d >> 3)) & 7); }
 
-// One block's K and V pieces of a thread, as fp16 (8 halfs per uint4).
-struct pa_stage_regs {
-    uint4 k0, k1;  // key tid / 8: dims (tid % 8) * 8 .. + 7 and 64 + (tid % 8) * 8 .. + 7
+// One block's K and V pieces of a thread as they come from the cache (an f32 cache is rounded when the pieces go to
+// LDS, after the block in between has been multiplied: the loads stay in flight meanwhile).
+template <bool KV16>
+struct pa_stage_regs;
+template <>
+struct pa_stage_regs<true> {
+    uint4 k0, k1;  // key t / 8 of the block: dims (t % 8) * 8 .. + 7 and 64 + (t % 8) * 8 .. + 7   (t = tid % 256)
     uint4 va, vb;  // two neighbouring keys: dims (lane % 16) * 8 .. + 7
+    __device__ __forceinline__ void load(uint4 &dst, const void *base, int64_t elem) {
+        dst = *reinterpret_cast<const uint4 *>(static_cast<const _Float16 *>(base) + elem);
+    }
+    __device__ __forceinline__ uint4 half8(const uint4 &v) const { return v; }
+};
+template <>
+struct pa_stage_regs<false> {
+    struct f8 {
+        float4 lo, hi;
+    };
+    f8 k0, k1, va, vb;
+    __device__ __forceinline__ void load(f8 &dst, const void *base, int64_t elem) {
+        const float4 *p = reinterpret_cast<const float4 *>(static_cast<const float *>(base) + elem);
+        dst.lo = p[0], dst.hi = p[1];
+    }
+    __device__ __forceinline__ uint4 half8(const f8 &v) const { return pa_pack8(v.lo, v.hi); }
 };
 
-template <bool KV16>
-__device__ __forceinline__ uint4 pa_load8(const void *base, int64_t elem, bool live) {
-    if (!live) return make_uint4(0, 0, 0, 0);
-    if (KV16) return *reinterpret_cast<const uint4 *>(static_cast<const _Float16 *>(base) + elem);
-    const float4 *p = reinterpret_cast<const float4 *>(static_cast<const float *>(base) + elem);
-    return pa_pack8(p[0], p[1]);
+// Block `blk` (32 keys) of the cache: the 256 threads of one half of the workgroup fetch it (t = tid % 256).  Keys
+// from kend on are not part of the walk (and may lie past the end of the cache): their loads are pointed at key
+// kend - 1, so that every load is unconditional, and pa_store replaces what they bring by zeros.
+__device__ __forceinline__ int pa_k_key(int blk, int t) { return blk * PA_BK + (t >> 3); }
+__device__ __forceinline__ int pa_v_key(int blk, int t) {
+    const int wv = t >> 6, w = (t & 63) >> 4;
+    return blk * PA_BK + ((w & 2) ? 16 : 0) + 4 * wv + 2 * (w & 1);
 }
 
 template <bool KV16>
-__device__ __forceinline__ void pa_fetch(pa_stage_regs &s, const pa_args &a, int head, int kb, int kend, int tid) {
+__device__ __forceinline__ void pa_fetch(pa_stage_regs<KV16> &s, const pa_args &a, int head, int blk, int kend, int t) {
     const int64_t E = (int64_t)a.n_head * PA_D;
     {
-        const int key = kb * PA_BK + (tid >> 3), piece = tid & 7;
-        const int64_t at = key * E + (int64_t)head * PA_D + piece * 8;
-        s.k0 = pa_load8<KV16>(a.kc, at, key < kend);
-        s.k1 = pa_load8<KV16>(a.kc, at + 64, key < kend);
+        const int key = min(pa_k_key(blk, t), kend - 1);
+        const int64_t at = key * E + (int64_t)head * PA_D + (t & 7) * 8;
+        s.load(s.k0, a.kc, at);
+        s.load(s.k1, a.kc, at + 64);
     }
     {
-        const int wave = tid >> 6, lane = tid & 63, w = lane >> 4, dg = lane & 15;
-        const int key = kb * PA_BK + ((w & 2) ? 16 : 0) + 4 * wave + 2 * (w & 1);
-        const int64_t at = key * E + (int64_t)head * PA_D + dg * 8;
-        // keys past the last one in use are zeros: their probabilities are zero, and 0 * (whatever the cache holds
-        // there) must not become NaN
-        s.va = pa_load8<KV16>(a.vc, at, key < kend);
-        s.vb = pa_load8<KV16>(a.vc, at + E, key + 1 < kend);
+        const int key = pa_v_key(blk, t);
+        const int64_t col = (int64_t)head * PA_D + (t & 15) * 8;
+        s.load(s.va, a.vc, min(key, kend - 1) * E + col);
+        s.load(s.vb, a.vc, min(key + 1, kend - 1) * E + col);
     }
 }
 
-__device__ __forceinline__ void pa_store(const pa_stage_regs &s, unsigned char *stage, int tid) {
+__device__ __forceinline__ uint4 pa_keep(const uint4 v, bool live) {
+    return make_uint4(live ? v.x : 0u, live ? v.y : 0u, live ? v.z : 0u, live ? v.w : 0u);
+}
+
+template <bool KV16>
+__device__ __forceinline__ void pa_store(const pa_stage_regs<KV16> &s, unsigned char *dst, int blk, int kend, int t) {
     {
-        unsigned char *row = stage + (tid >> 3) * PA_KROW + (tid & 7) * 16;
-        *reinterpret_cast<uint4 *>(row) = s.k0;
-        *reinterpret_cast<uint4 *>(row + 128) = s.k1;
+        // keys past the last one in use are zeros: their probabilities are zero, and 0 * (whatever a cache holds
+        // there) must not become NaN
+        const bool live = pa_k_key(blk, t) < kend;
+        unsigned char *row = dst + (t >> 3) * PA_KROW + (t & 7) * 16;
+        *reinterpret_cast<uint4 *>(row) = pa_keep(s.half8(s.k0), live);
+        *reinterpret_cast<uint4 *>(row + 128) = pa_keep(s.half8(s.k1), live);
     }
     {
-        const int wave = tid >> 6, lane = tid & 63, w = lane >> 4, dg = lane & 15;
-        unsigned char *vt = stage + PA_KBYTES + (4 * wave + w) * 4;  // the pair of slots 8 * wave + 2 * w, + 1
-        const uint32_t a[4] = {s.va.x, s.va.y, s.va.z, s.va.w}, b[4] = {s.vb.x, s.vb.y, s.vb.z, s.vb.w};
+        const int wv = t >> 6, lane = t & 63, w = lane >> 4, dg = lane & 15;
+        const int key = pa_v_key(blk, t);
+        unsigned char *vt = dst + PA_KBYTES + (4 * wv + w) * 4;  // the pair of slots 8 * wv + 2 * w, + 1
+        const uint4 va = pa_keep(s.half8(s.va), key < kend), vb = pa_keep(s.half8(s.vb), key + 1 < kend);
+        const uint32_t a[4] = {va.x, va.y, va.z, va.w}, b[4] = {vb.x, vb.y, vb.z, vb.w};
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const uint32_t lo = (e & 1) ? (a[e >> 1] >> 16) : (a[e >> 1] & 0xffffu);
@@ -123,17 +153,20 @@ __device__ __forceinline__ void pa_store(const pa_stage_regs &s, unsigned char *
 
 template <int QT, bool KV16, bool PANEL>
 __global__ __launch_bounds__(PA_THREADS) void attn_prefill_kernel(const pa_args a) {
-    __shared__ __align__(16) unsigned char lds[2 * PA_STAGE];
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // two stages of two blocks: [K 32 x 272 | V^T 128 x 80]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int half = wave >> 2;   // which block of a stage this wave multiplies (and helps to fetch)
+    const int wq = wave & 3;      // which queries of the workgroup it owns
+    const int t = tid & 255;
     constexpr int BM = 64 * QT;
     const int head = blockIdx.x % a.n_head;
     const int tile = a.tiles - 1 - blockIdx.x / a.n_head;  // long walks first
     const int m0 = tile * BM;
     const int m_last = (m0 + BM < a.n ? m0 + BM : a.n) - 1;   // the workgroup's last live query
     const int kend = a.n_past + m_last + 1;                   // keys it may see
-    const int nblk = (kend + PA_BK - 1) / PA_BK;
+    const int nstage = (kend + 2 * PA_BK - 1) / (2 * PA_BK);
     const int64_t E = (int64_t)a.n_head * PA_D;
-    const int mw0 = m0 + wave * 16 * QT;                      // the wave's first query
+    const int mw0 = m0 + wq * 16 * QT;                        // the wave's first query
 
     // Q^T fragments, scaled: for query tile qt and chunk c, dims c * 32 + g * 8 .. + 7 of query mw0 + qt * 16 + r
     half8_t qf[QT][4];
@@ -160,19 +193,19 @@ __global__ __launch_bounds__(PA_THREADS) void attn_prefill_kernel(const pa_args 
     for (int qt = 0; qt < QT; qt++) {
         m_run[qt] = -INFINITY, l_run[qt] = 0.0f;
 #pragma unroll
-        for (int t = 0; t < 8; t++) acc[qt][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int tt = 0; tt < 8; tt++) acc[qt][tt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    pa_stage_regs st;
-    pa_fetch<KV16>(st, a, head, 0, kend, tid);
-    pa_store(st, lds, tid);
+    pa_stage_regs<KV16> st;
+    pa_fetch<KV16>(st, a, head, half, kend, t);
+    pa_store<KV16>(st, lds + half * PA_BLOCK, half, kend, t);
     __syncthreads();
 
-    for (int kb = 0; kb < nblk; kb++) {
-        const bool more = kb + 1 < nblk;
-        if (more) pa_fetch<KV16>(st, a, head, kb + 1, kend, tid);
-        const unsigned char *ks = lds + (kb & 1) * PA_STAGE, *vt = ks + PA_KBYTES;
-        const int key0 = kb * PA_BK;
+    for (int sg = 0; sg < nstage; sg++) {
+        const bool more = sg + 1 < nstage;
+        if (more) pa_fetch<KV16>(st, a, head, (sg + 1) * 2 + half, kend, t);
+        const unsigned char *ks = lds + (sg & 1) * PA_STAGE + half * PA_BLOCK, *vt = ks + PA_KBYTES;
+        const int key0 = (sg * 2 + half) * PA_BK;
         // the wave's last query sees keys up to n_past + mw0 + 16 * QT - 1: blocks behind that are nothing to it
         if (key0 <= a.n_past + mw0 + 16 * QT - 1) {
             float4_t s[QT][2];
@@ -203,40 +236,68 @@ __global__ __launch_bounds__(PA_THREADS) void attn_prefill_kernel(const pa_args 
                 float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
                 mx = fmaxf(mx, __shfl_xor(mx, 16));
                 mx = fmaxf(mx, __shfl_xor(mx, 32));
-                // key 0 is visible to every query, so the maximum is finite from the first block on
+                // a query that has seen no key yet (the second block of a stage can lie behind its mask) keeps -inf as
+                // its maximum; the exponentials then take 0 as their reference and come out as exact zeros
                 const float m_new = fmaxf(m_run[qt], mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_ref);
                 m_run[qt] = m_new;
                 float sum = 0.0f;
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
-                    v[i] = __builtin_amdgcn_exp2f(v[i] - m_new);
+                    v[i] = __builtin_amdgcn_exp2f(v[i] - m_ref);
                     sum += v[i];
                 }
                 l_run[qt] = l_run[qt] * alpha + sum;
                 pf[qt] = __builtin_bit_cast(half8_t, make_uint4(pa_pack(v[0], v[1]), pa_pack(v[2], v[3]), pa_pack(v[4], v[5]),
                                                                 pa_pack(v[6], v[7])));
 #pragma unroll
-                for (int t = 0; t < 8; t++) acc[qt][t] *= alpha;
+                for (int tt = 0; tt < 8; tt++) acc[qt][tt] *= alpha;
             }
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
-                const half8_t vf = *reinterpret_cast<const half8_t *>(vt + pa_vrow(t * 16 + r) * PA_VROW + g * 16);
+            for (int tt = 0; tt < 8; tt++) {
+                const half8_t vf = *reinterpret_cast<const half8_t *>(vt + pa_vrow(tt * 16 + r) * PA_VROW + g * 16);
 #pragma unroll
                 for (int qt = 0; qt < QT; qt++)
-                    acc[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[qt], acc[qt][t], 0, 0, 0);
+                    acc[qt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[qt], acc[qt][tt], 0, 0, 0);
             }
         }
-        if (more) pa_store(st, lds + ((kb + 1) & 1) * PA_STAGE, tid);
+        if (more) pa_store<KV16>(st, lds + ((sg + 1) & 1) * PA_STAGE + half * PA_BLOCK, (sg + 1) * 2 + half, kend, t);
         __syncthreads();
     }
 
+    // The two waves that own the same queries (one walked the first block of every stage, the other the second) meet:
+    // the second hands over maximum, sum and output through LDS (free after the last barrier), the first merges.
+    float *xch = reinterpret_cast<float *>(lds) + wq * (QT * 34 * 64) + lane;
+    if (half == 1) {
+#pragma unroll
+        for (int qt = 0; qt < QT; qt++) {
+            float *x = xch + qt * 34 * 64;
+            x[0] = m_run[qt], x[64] = l_run[qt];
+#pragma unroll
+            for (int tt = 0; tt < 8; tt++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) x[(2 + tt * 4 + j) * 64] = acc[qt][tt][j];
+        }
+    }
+    __syncthreads();
+    if (half == 1) return;
+
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
-        float l = l_run[qt];
+        const float *x = xch + qt * 34 * 64;
+        // the first wave has seen key 0, so the common maximum is finite
+        const float m2 = x[0], m_all = fmaxf(m_run[qt], m2);
+        const float a1 = __builtin_amdgcn_exp2f(m_run[qt] - m_all), a2 = __builtin_amdgcn_exp2f(m2 - m_all);
+        float l = l_run[qt] * a1 + x[64] * a2;
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
         const float inv = 1.0f / l;
+        float4_t o[8];
+#pragma unroll
+        for (int tt = 0; tt < 8; tt++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[tt][j] = (acc[qt][tt][j] * a1 + x[(2 + tt * 4 + j) * 64] * a2) * inv;
         const int m = mw0 + qt * 16 + r;
         if (PANEL) {
             // element (m, k) of the panel: tile (m / 16, k / 32) of 1 KB, 16-byte piece ((k % 32) / 8) * 16 + m % 16
@@ -245,32 +306,34 @@ __global__ __launch_bounds__(PA_THREADS) void attn_prefill_kernel(const pa_args 
                 unsigned char *row = reinterpret_cast<unsigned char *>(a.panel) + ((int64_t)(m >> 4) * (E >> 5) + head * 4) * 1024 +
                                      (m & 15) * 16 + (g & 1) * 8;
 #pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    uint2 o = make_uint2(0, 0);  // rows past n are zeros in a panel
-                    if (m < a.n) o = make_uint2(pa_pack(acc[qt][t][0] * inv, acc[qt][t][1] * inv), pa_pack(acc[qt][t][2] * inv, acc[qt][t][3] * inv));
-                    *reinterpret_cast<uint2 *>(row + (t >> 1) * 1024 + ((t & 1) * 2 + (g >> 1)) * 256) = o;
+                for (int tt = 0; tt < 8; tt++) {
+                    uint2 w2 = make_uint2(0, 0);  // rows past n are zeros in a panel
+                    if (m < a.n) w2 = make_uint2(pa_pack(o[tt][0], o[tt][1]), pa_pack(o[tt][2], o[tt][3]));
+                    *reinterpret_cast<uint2 *>(row + (tt >> 1) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256) = w2;
                 }
             }
         } else if (m < a.n) {
             float *row = a.out + m * E + (int64_t)head * PA_D + g * 4;
 #pragma unroll
-            for (int t = 0; t < 8; t++)
-                *reinterpret_cast<float4 *>(row + t * 16) =
-                    make_float4(acc[qt][t][0] * inv, acc[qt][t][1] * inv, acc[qt][t][2] * inv, acc[qt][t][3] * inv);
+            for (int tt = 0; tt < 8; tt++) *reinterpret_cast<float4 *>(row + tt * 16) = make_float4(o[tt][0], o[tt][1], o[tt][2], o[tt][3]);
         }
     }
 }
 
+template <int QT, bool KV16, bool PANEL>
+hipError_t pa_launch_one(galois_hip_ctx *ctx, const pa_args &a) {
+    const hipError_t e = hipFuncSetAttribute((const void *)attn_prefill_kernel<QT, KV16, PANEL>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, PA_LDS);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((attn_prefill_kernel<QT, KV16, PANEL>), dim3((unsigned)(a.tiles * a.n_head)), dim3(PA_THREADS), PA_LDS,
+                       ctx->stream, a);
+    return hipSuccess;
+}
+
 template <int QT>
-void pa_launch(galois_hip_ctx *ctx, const pa_args &a, bool kv16, bool panel) {
-    const dim3 grid((unsigned)(a.tiles * a.n_head)), block(PA_THREADS);
-    if (kv16) {
-        if (panel) hipLaunchKernelGGL((attn_prefill_kernel<QT, true, true>), grid, block, 0, ctx->stream, a);
-        else hipLaunchKernelGGL((attn_prefill_kernel<QT, true, false>), grid, block, 0, ctx->stream, a);
-    } else {
-        if (panel) hipLaunchKernelGGL((attn_prefill_kernel<QT, false, true>), grid, block, 0, ctx->stream, a);
-        else hipLaunchKernelGGL((attn_prefill_kernel<QT, false, false>), grid, block, 0, ctx->stream, a);
-    }
+hipError_t pa_launch(galois_hip_ctx *ctx, const pa_args &a, bool kv16, bool panel) {
+    if (kv16) return panel ? pa_launch_one<QT, true, true>(ctx, a) : pa_launch_one<QT, true, false>(ctx, a);
+    return panel ? pa_launch_one<QT, false, true>(ctx, a) : pa_launch_one<QT, false, false>(ctx, a);
 }
 
 int32_t pa_entry(galois_hip_ctx *ctx, const float *q, const void *k_cache, const void *v_cache, bool kv16, float *out, void *out_panel,
@@ -293,8 +356,8 @@ int32_t pa_entry(galois_hip_ctx *ctx, const float *q, const void *k_cache, const
     const int qt = wg64 > (int64_t)ctx->n_cu * 4 ? 2 : 1;
     a.tiles = (n_tokens + 64 * qt - 1) / (64 * qt);
     GH_REQUIRE(ctx, (int64_t)a.tiles * n_head < ((int64_t)1 << 31), GALOIS_HIP_E_SHAPE, "attn_prefill: too many workgroups");
-    if (qt == 2) pa_launch<2>(ctx, a, kv16, out_panel != nullptr);
-    else pa_launch<1>(ctx, a, kv16, out_panel != nullptr);
+    const hipError_t e = qt == 2 ? pa_launch<2>(ctx, a, kv16, out_panel != nullptr) : pa_launch<1>(ctx, a, kv16, out_panel != nullptr);
+    if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
     GH_LAUNCH_CHECK(ctx, "attn_prefill");
 }
 
