@@ -280,6 +280,12 @@ class Device:
         self._check(fn(self._ctx, arr, _ptr(k_cache), _ptr(v_cache), _ptr(out), n_head, head_dim, n_past, _ptr(pos),
                        freq_scale, theta_scale, scale, head_major_n_ctx))
 
+    def mul_mat_q4_0_f16_panel_add(self, W, panel, residual, Y, K, N, M, workspace=None, workspace_bytes=0):
+        """Y = residual + W . panel (residual may be None); with a workspace of 2 * M * N floats a matrix too narrow
+        for the device is multiplied as two shares of k."""
+        self._check(self._lib.galois_hip_mul_mat_q4_0_f16_panel_add(self._ctx, _ptr(W), _ptr(panel), _ptr(residual), _ptr(Y), K, N, M,
+                                                                    _ptr(workspace), workspace_bytes))
+
     def attn_prefill(self, q, k_cache, v_cache, out, out_panel, n_head, head_dim, n_tokens, n_past, scale, kv_f16=False):
         """Causal attention of n_tokens rows of q over caches that already hold positions 0 .. n_past + n_tokens - 1;
         the result goes to out (f32) or out_panel (fp16 panel), the other is None."""

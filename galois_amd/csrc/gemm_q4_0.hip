@@ -403,18 +403,19 @@ __device__ __forceinline__ void gemm_stage_write(const gemm_stage_regs<GN> &r, _
 // Barrier protocol (both kinds of wave meet every one): R after the first raw piece is parked,
 // then barrier t after stage t is written, for t = 0 .. nslots-1.  Stage t goes to buffer t % 3.
 template <int GN>
-__device__ __forceinline__ void gemm_producer(_Float16 *smem, const gemm_mats &mats, int K, int n0) {
+__device__ __forceinline__ void gemm_producer(_Float16 *smem, const gemm_mats &mats, int K, int n0, int sup0, int nsuper) {
     constexpr int GB_HALFS = gemm_cfg<GN>::B_HALFS, GRAW_BYTES = gemm_cfg<GN>::RAW_BYTES;
     const int p = threadIdx.x - 256;
-    const int nslots = K / 64;            // stages; a multiple of 4 (K % 256 == 0)
-    const int nsuper = nslots / 4;
-    const size_t wrow_bytes = (size_t)nslots * 36;
+    // the workgroup's share of k: pieces sup0 .. sup0 + nsuper - 1 of 256 weights (four stages) of every row
+    const size_t wrow_bytes = (size_t)(K / 64) * 36;
     uint8_t *raw0 = reinterpret_cast<uint8_t *>(smem + GNBUF * GB_HALFS);
     uint8_t *raw1 = raw0 + GRAW_BYTES;
 
     gemm_raw_regs<GN> rr;
     const uint8_t *rowp[gemm_cfg<GN>::RAW_PER_THREAD];
     gemm_raw_rows<GN>(mats, wrow_bytes, n0, p, rowp);
+#pragma unroll
+    for (int i = 0; i < gemm_cfg<GN>::RAW_PER_THREAD; i++) rowp[i] += (size_t)sup0 * GRAW_STRIDE;
     gemm_load_raw<GN>(rowp, 0, rr);
     GEMM_VMWAIT(0);
     gemm_store_raw(raw0, p, rr);
@@ -481,10 +482,12 @@ __device__ __forceinline__ void gemm_load_a1(u32x4_t &dst, const _Float16 *xs, u
 #define GEMM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
 template <int NF, int GN>
 __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float16 *__restrict__ Xh,
-                                              const gemm_mats &mats, int K, int M, int m0, int n0, int wm, int ncol0) {
+                                              const gemm_mats &mats, int K, int M, int m0, int n0, int wm, int ncol0,
+                                              int nslots, size_t y_off) {
+    // Xh: the panel advanced to the workgroup's first k-block; nslots: its stages; y_off: where its results go,
+    // relative to Y (a workgroup that holds one share of k of several writes a partial result)
     constexpr int GB_HALFS = gemm_cfg<GN>::B_HALFS;
     const int lane = threadIdx.x & 63;
-    const int nslots = K / 64;
     float4_t acc[4][NF];
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -607,6 +610,7 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
             Y = ge ? mats.Y[t] : Y, N = ge ? mats.N[t] : N, first = ge ? mats.col0[t] : first;
         }
         const int nl = n - first;
+        Y += y_off;
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -619,48 +623,88 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
 
 template <int GN>
 __global__ __launch_bounds__(512) void gemm_q4_0_mfma(const gemm_mats mats, const _Float16 *__restrict__ Xh, int K, int M,
-                                                      int n_tiles, int m_tiles) {
+                                                      int n_tiles, int m_tiles, int splits, size_t split_stride) {
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[];  // [3] B stage | [2] raw | pad
-    // XCD-aware tile order: blockIdx % 8 is the XCD; consecutive tiles (same X panel) go to one XCD
-    const int total = n_tiles * m_tiles;
+    // XCD-aware tile order: blockIdx % 8 is the XCD; consecutive tiles (same X panel, same share of k) go to one XCD
+    const int total = n_tiles * m_tiles * splits;
     const int per_xcd = (total + 7) >> 3;
     const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (tile >= total) return;
-    const int mt = tile / n_tiles, nt = tile - mt * n_tiles;
+    const int mts = tile / n_tiles, nt = tile - mts * n_tiles;
+    const int sp = mts / m_tiles, mt = mts - sp * m_tiles;
     const int m0 = mt * GM, n0 = nt * GN;
+    // share sp of k: whole pieces of 256 (four stages), as evenly as they divide; its results lie split_stride
+    // floats after the previous share's
+    const int nsuper_all = K / 256;
+    const int sup0 = (int)((int64_t)sp * nsuper_all / splits), sup1 = (int)((int64_t)(sp + 1) * nsuper_all / splits);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (wave >= 4)
-        gemm_producer<GN>(smem, mats, K, n0);
-    else  // four consumer waves stacked in M, each 64 rows x GN columns
-        gemm_consumer<GN / 16, GN>(smem, Xh, mats, K, M, m0, n0, wave, 0);
+        gemm_producer<GN>(smem, mats, K, n0, sup0, sup1 - sup0);
+    else  // four consumer waves stacked in M, each 64 rows x GN columns; a piece of 256 is 8 KB of a row group's panel
+        gemm_consumer<GN / 16, GN>(smem, Xh + (size_t)sup0 * 4096, mats, K, M, m0, n0, wave, 0, (sup1 - sup0) * 4,
+                                   (size_t)sp * split_stride);
+}
+
+// The pass behind a product with a residual: y = p (+ the second share of k, stride4 float4s on, when stride4 != 0)
+// (+ r), four floats per thread.  y may be p (a product already in place) or r (the residual stream updated in place):
+// every thread reads its own four elements before it writes them.  Measured against adding the residual where the
+// product's tiles are stored: the separate pass is faster (512 x 4096 x 11008: 58.6 against 68.0 us), since the
+// tiles' scattered 4-byte reads of the residual sit at the end of every workgroup with nothing left to hide them.
+__global__ __launch_bounds__(256) void gemm_sum_pass(const float4 *p, const float4 *r, float4 *y, int64_t n4, int64_t stride4) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    float4 o = p[i];
+    if (stride4) {
+        const float4 b = p[i + stride4];
+        o = make_float4(o.x + b.x, o.y + b.y, o.z + b.z, o.w + b.w);
+    }
+    if (r) {
+        const float4 c = r[i];
+        o = make_float4(o.x + c.x, o.y + c.y, o.z + c.z, o.w + c.w);
+    }
+    __builtin_nontemporal_store(float4_t{o.x, o.y, o.z, o.w}, reinterpret_cast<float4_t *>(y + i));
+}
+
+// The same for a result whose size is not a multiple of four floats.
+__global__ __launch_bounds__(256) void gemm_sum_tail(const float *p, const float *r, float *y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = p[i] + r[i];
 }
 
 // Launch of one tile width.
 template <int GN>
-int32_t gemm_launch(galois_hip_ctx *ctx, const gemm_mats &mats, const _Float16 *Xh, int K, int M) {
+int32_t gemm_launch(galois_hip_ctx *ctx, const gemm_mats &mats, const _Float16 *Xh, int K, int M, int splits = 1,
+                    size_t split_stride = 0) {
     const int n_tiles = (mats.n_total + GN - 1) / GN;
     const int m_tiles = (M + GM - 1) / GM;
-    const int total = n_tiles * m_tiles;
+    const int total = n_tiles * m_tiles * splits;
     const int grid = ((total + 7) / 8) * 8;
     const size_t lds = gemm_cfg<GN>::LDS_BYTES;
     // the attribute lives with the function on the current device: set per launch (a table lookup), which is right
     // for every device and every thread without any flag of our own
     hipError_t e = hipFuncSetAttribute((const void *)gemm_q4_0_mfma<GN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return gh_hip(ctx, e, "hipFuncSetAttribute(LDS size)");
-    hipLaunchKernelGGL(gemm_q4_0_mfma<GN>, dim3(grid), dim3(512), lds, ctx->stream, mats, Xh, K, M, n_tiles, m_tiles);
+    hipLaunchKernelGGL(gemm_q4_0_mfma<GN>, dim3(grid), dim3(512), lds, ctx->stream, mats, Xh, K, M, n_tiles, m_tiles, splits,
+                       split_stride);
     return GALOIS_HIP_OK;
 }
 
 // Tile width by how many workgroups it gives the device.  Cost model: rounds of workgroups over the CUs
 // times the relative cost of a k-stage (a 48-column stage has half the matrix instructions and half
 // the dequantisation of a 96-column one but the same barriers and A requests: ~0.65).
-int32_t gemm_launch_any(galois_hip_ctx *ctx, gemm_mats mats, int n_mats, const _Float16 *Xh, int K, int M) {
+// Numbers the columns of the first n_mats matrices through (col0, n_total).
+void gemm_concat(gemm_mats &mats, int n_mats) {
     int64_t cols = 0;
     for (int j = 0; j < GEMM_MAX_MATS; j++) {
         mats.col0[j] = j < n_mats ? (int32_t)cols : 0x7FFFFFFF;
         if (j < n_mats) cols += mats.N[j];
     }
     mats.n_total = (int32_t)cols;
+}
+
+int32_t gemm_launch_any(galois_hip_ctx *ctx, gemm_mats mats, int n_mats, const _Float16 *Xh, int K, int M) {
+    gemm_concat(mats, n_mats);
+    const int64_t cols = mats.n_total;
     const int64_t m_tiles = (M + GM - 1) / GM;
     const int64_t wg96 = (cols + 95) / 96 * m_tiles, wg48 = (cols + 47) / 48 * m_tiles;
     const int64_t cus = ctx->n_cu > 0 ? ctx->n_cu : 256;
@@ -804,4 +848,59 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel(galois_hip_ctx *ctx, const 
     const int32_t st = gemm_launch_any(ctx, mats, n_items, (const _Float16 *)panel, K, M);
     if (st != GALOIS_HIP_OK) return st;
     GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel launch");
+}
+
+// One matrix against the panel with a residual added, and the k-split shape for matrices too narrow to fill the device.
+extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, const void *W, const void *panel, const float *residual,
+                                                         float *Y, int32_t K, int32_t N, int32_t M, void *workspace,
+                                                         int64_t workspace_bytes) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, W && panel && Y, GALOIS_HIP_E_NULL, "mul_mat_q4_0_f16_panel_add");
+    GH_REQUIRE(ctx, gemm_panel_shape_ok(K, M) && N > 0 && (int64_t)M * N < ((int64_t)1 << 31), GALOIS_HIP_E_SHAPE,
+               "mul_mat_q4_0_f16_panel_add: K a positive multiple of 256, (M + 16) * K below 2^31, N positive, M * N below 2^31");
+    GH_REQUIRE(ctx, gh_aligned(W, 16) && gh_aligned(panel, 16) && gh_aligned(Y, 16) && gh_aligned(residual, 16) && gh_aligned(workspace, 16),
+               GALOIS_HIP_E_ALIGN, "mul_mat_q4_0_f16_panel_add: 16-byte aligned operands");
+    GH_REQUIRE(ctx, workspace_bytes >= 0, GALOIS_HIP_E_SHAPE, "mul_mat_q4_0_f16_panel_add: workspace_bytes");
+    GH_BIND(ctx);
+    gemm_mats mats = {};
+    mats.W[0] = (const uint8_t *)W, mats.Y[0] = Y, mats.N[0] = N;
+    // Two shares of k, each a workgroup of 64 columns, when that fills the device better than whole-k tiles do: the
+    // cost model of gemm_launch_any (rounds of workgroups x cost of a stage x stages; a 64-column stage on a full
+    // device at 0.75 of a 96-column one) plus the pass that adds the two partial results, which costs about fourteen
+    // stages per 2^21 results.  Measured at M = 512 on 256 CUs: 11008 -> 4096 70.3 -> 54.8 us, 4096 -> 4096 32.5 -> 30.2 us
+    // (both with the residual), and the shapes the model leaves whole are slower when forced into shares.
+    const int64_t m_tiles = (M + GM - 1) / GM, cus = ctx->n_cu > 0 ? ctx->n_cu : 256, stages = K / 64;
+    const int64_t wg96 = ((int64_t)N + 95) / 96 * m_tiles, wg48 = ((int64_t)N + 47) / 48 * m_tiles, wg64x2 = ((int64_t)N + 63) / 64 * m_tiles * 2;
+    const int64_t mn = (int64_t)M * N;
+    const double c96 = (double)((wg96 + cus - 1) / cus) * stages, c48 = 0.65 * (double)((wg48 + cus - 1) / cus) * stages;
+    const double c64x2 = 0.75 * (double)((wg64x2 + cus - 1) / cus) * (stages / 2 + 2) + 14.0 * (double)mn / (double)(1 << 21);
+    const bool can_split = workspace && workspace_bytes >= 2 * mn * (int64_t)sizeof(float) && K >= 512 && mn % 4 == 0;
+    const dim3 sum_grid((unsigned)((mn / 4 + 255) / 256));
+    if (can_split && c64x2 < c96 && c64x2 < c48) {
+        mats.Y[0] = static_cast<float *>(workspace);
+        gemm_concat(mats, 1);
+        const int32_t st = gemm_launch<64>(ctx, mats, (const _Float16 *)panel, K, M, 2, (size_t)mn);
+        if (st != GALOIS_HIP_OK) return st;
+        hipLaunchKernelGGL(gemm_sum_pass, sum_grid, dim3(256), 0, ctx->stream, static_cast<const float4 *>(workspace),
+                           reinterpret_cast<const float4 *>(residual), reinterpret_cast<float4 *>(Y), mn / 4, mn / 4);
+    } else {
+        // the product needs a place of its own while the residual is still to be read: Y unless Y is the residual
+        float *prod = Y;
+        if (residual == Y) {
+            GH_REQUIRE(ctx, workspace && workspace_bytes >= mn * (int64_t)sizeof(float), GALOIS_HIP_E_UNSUPPORTED,
+                       "mul_mat_q4_0_f16_panel_add: Y may be the residual only with a workspace of M * N floats or more");
+            prod = static_cast<float *>(workspace);
+        }
+        mats.Y[0] = prod;
+        const int32_t st = gemm_launch_any(ctx, mats, 1, (const _Float16 *)panel, K, M);
+        if (st != GALOIS_HIP_OK) return st;
+        if (residual) {
+            if (mn % 4 == 0)
+                hipLaunchKernelGGL(gemm_sum_pass, sum_grid, dim3(256), 0, ctx->stream, reinterpret_cast<const float4 *>(prod),
+                                   reinterpret_cast<const float4 *>(residual), reinterpret_cast<float4 *>(Y), mn / 4, (int64_t)0);
+            else
+                hipLaunchKernelGGL(gemm_sum_tail, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, ctx->stream, prod, residual, Y, mn);
+        }
+    }
+    GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel_add launch");
 }

@@ -55,11 +55,12 @@ class LlamaDecoder {
     // norms and the SwiGLU write directly (q | k | v and gate | up one launch each), rope_custom over all positions,
     // the n new rows of both caches appended at once, scores = K^T Q and out = V P per head on the matrix cores with
     // a causal soft_max between them (heads of 128: galois_attn_prefill instead, one launch that writes the panel of
-    // the output projection; f32 caches then also receive the rotated keys and the values directly).  Afterwards the caches hold positions 0 .. n_past + n - 1 and logits() the last
+    // the output projection; f32 caches receive the rotated keys and the values directly); the output and down
+    // projections add the residual stream where they store (galois_matmul_panel_add).  Afterwards the caches hold positions 0 .. n_past + n - 1 and logits() the last
     // token's.  n_embd and n_ff must be multiples of 256; caches [n_embd, n_ctx] (not head-major), f32 or f16.
     // Intermediates are sized for the largest n and n_past + n seen so far (this call allocates when they grow).
     GResult prefill(const int32_t *tokens, size_t n, int32_t n_past);
-    size_t ops_per_prefill() const { return n_prefill_ops_; }
+    size_t ops_per_prefill() const { return n_prefill_ops_; }  // library calls of the last prefill (a call is one or two launches)
     const Tensor &logits() const { return logits_; }
     const LlamaHParams &hparams() const { return hp_; }
     size_t ops_per_step() const { return n_ops_; }
@@ -80,7 +81,7 @@ class LlamaDecoder {
     Tensor ssq_, ssq1_;  // partial sums of squares of x and x1 (fused = 4)
     struct Prefill {  // intermediates of prefill(), for up to `rows` tokens attending over up to `keys` positions
         size_t rows = 0, keys = 0;
-        Tensor tok, pos, x, x1, t, q, k, v, qr, kr, q3, s, p, o, ao, g, u, panel_e, panel_f;
+        Tensor tok, pos, x, x1, q, k, v, qr, kr, q3, s, p, o, ao, g, u, panel_e, panel_f, split_ws;
     };
     GResult prefill_buffers(size_t n, size_t keys);
     Prefill pf_;
@@ -121,6 +122,10 @@ struct PanelMatmulItem {
     Tensor *dst = nullptr;
 };
 GResult galois_matmul_panel(const std::vector<PanelMatmulItem> &items, const Tensor &panel, size_t K, size_t M);
+// dst = residual + w . panel (galois_hip_mul_mat_q4_0_f16_panel_add); residual may be null or dst.  workspace: an F32
+// tensor the call may overwrite (2 * N * M elements let a narrow matrix run as two shares of k), or null.
+GResult galois_matmul_panel_add(const Tensor &w, const Tensor &panel, const Tensor *residual, Tensor &dst, size_t K, size_t M,
+                                Tensor *workspace);
 
 // Attention of one decode step in one launch (galois_hip_attn_decode_f32): rope_custom of q and k at position
 // pos[0] = n_past, append of k and v to row n_past of the caches ([n_embd, n_ctx], both f32 or both f16), scores = K^T q scaled

@@ -84,6 +84,31 @@ GResult galois_matmul_panel(const std::vector<PanelMatmulItem> &items, const Ten
     return dev->check(galois_hip_mul_mat_q4_0_f16_panel(dev->ctx(), it, (int32_t)items.size(), panel.data(), (int32_t)K, (int32_t)M));
 }
 
+GResult galois_matmul_panel_add(const Tensor &w, const Tensor &panel, const Tensor *residual, Tensor &dst, size_t K, size_t M,
+                                Tensor *workspace) {
+    if (!panel.device().is_gpu() || panel.dtype() != GGmlType::F16 || panel.dim().elem_count() < galois_panel_elems(K, M))
+        return err(GError::ShapeError, "galois_matmul_panel_add: an F16 Gpu panel of galois_panel_elems(K, M) elements");
+    const auto &dev = panel.device().gpu;
+    for (const Tensor *t : {&w, (const Tensor *)&dst, residual, (const Tensor *)workspace})
+        if (t && (!t->device().is_gpu() || t->device().gpu != dev))
+            return err(GError::Unimplemented, "galois_matmul_panel_add: Gpu tensors on the panel's device");
+    if (w.dtype() != GGmlType::Q4_0 || dst.dtype() != GGmlType::F32 || !w.dim().ggml_is_contiguous(w.dtype()) ||
+        !dst.dim().ggml_is_contiguous(dst.dtype()))
+        return err(GError::Unimplemented, "galois_matmul_panel_add: a contiguous Q4_0 matrix and an F32 result");
+    const size_t N = w.dim().shape[1];
+    if (w.dim().shape[0] != K || w.dim().elem_count() != K * N || dst.dim().elem_count() != N * M)
+        return err(GError::ShapeError, "galois_matmul_panel_add: w [K, N], dst [N, M]");
+    if (residual && (residual->dtype() != GGmlType::F32 || !residual->dim().ggml_is_contiguous(residual->dtype()) ||
+                     residual->dim().elem_count() != N * M))
+        return err(GError::ShapeError, "galois_matmul_panel_add: residual F32 [N, M]");
+    if (workspace && (workspace->dtype() != GGmlType::F32 || !workspace->dim().ggml_is_contiguous(workspace->dtype())))
+        return err(GError::ShapeError, "galois_matmul_panel_add: workspace contiguous F32");
+    return dev->check(galois_hip_mul_mat_q4_0_f16_panel_add(
+        dev->ctx(), w.data(), panel.data(), residual ? (const float *)residual->data() : nullptr, (float *)dst.data(), (int32_t)K,
+        (int32_t)N, (int32_t)M, workspace ? workspace->data() : nullptr,
+        workspace ? (int64_t)(workspace->dim().elem_count() * sizeof(float)) : 0));
+}
+
 GResult galois_attn_prefill(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &dst, size_t n_head,
                             int32_t n_past, float scale) {
     for (const Tensor *t : {&q, &k_cache, &v_cache, (const Tensor *)&dst})
@@ -131,7 +156,7 @@ GResult LlamaDecoder::prefill_buffers(size_t n, size_t keys) {
     const GGmlType F32 = GGmlType::F32;
     G_TRY(mk(&b.tok, GGmlType::I32, dev_, rows));
     G_TRY(mk(&b.pos, GGmlType::I32, dev_, rows));
-    for (Tensor *t : {&b.x, &b.x1, &b.t, &b.q, &b.k, &b.v, &b.ao}) G_TRY(mk(t, F32, dev_, E, rows));
+    for (Tensor *t : {&b.x, &b.x1, &b.q, &b.k, &b.v, &b.ao}) G_TRY(mk(t, F32, dev_, E, rows));
     G_TRY(mk(&b.qr, F32, dev_, D, H, rows));
     G_TRY(mk(&b.kr, F32, dev_, D, H, rows));
     G_TRY(mk(&b.q3, F32, dev_, D, rows, H));
@@ -142,6 +167,7 @@ GResult LlamaDecoder::prefill_buffers(size_t n, size_t keys) {
     G_TRY(mk(&b.u, F32, dev_, F, rows));
     G_TRY(mk(&b.panel_e, GGmlType::F16, dev_, galois_panel_elems(E, rows)));
     G_TRY(mk(&b.panel_f, GGmlType::F16, dev_, galois_panel_elems(F, rows)));
+    G_TRY(mk(&b.split_ws, F32, dev_, 2 * E * rows));
     b.rows = rows, b.keys = kk;
     pf_ = std::move(b);
     return GError{};
@@ -161,12 +187,12 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
     Prefill &b = pf_;
     galois_hip_ctx *ctx = dev_.gpu->ctx();
     // views of the buffers at this call's n and L (the buffers may be larger)
-    Tensor tok, pos, x, x1, t, q, k, v, ao, qr, kr, q3, o, s, p, g, u;
+    Tensor tok, pos, x, x1, q, k, v, ao, qr, kr, q3, o, s, p, g, u;
     {
         const size_t one[1] = {n}, en[2] = {E, n}, fn[2] = {F, n}, dhn[3] = {D, H, n}, dnh[3] = {D, n, H}, lnh[3] = {L, n, H};
         G_TRY(b.tok.view(0, 1, one, &tok));
         G_TRY(b.pos.view(0, 1, one, &pos));
-        for (auto pr : {std::make_pair(&b.x, &x), std::make_pair(&b.x1, &x1), std::make_pair(&b.t, &t), std::make_pair(&b.q, &q),
+        for (auto pr : {std::make_pair(&b.x, &x), std::make_pair(&b.x1, &x1), std::make_pair(&b.q, &q),
                         std::make_pair(&b.k, &k), std::make_pair(&b.v, &v), std::make_pair(&b.ao, &ao)})
             G_TRY(pr.first->view(0, 2, en, pr.second));
         G_TRY(b.qr.view(0, 3, dhn, &qr));
@@ -253,14 +279,13 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
             }
             G_TRY(galois_to_panel(ao, b.panel_e)); ops++;
         }
-        G_TRY(galois_matmul_panel({{&l.wo, &t}}, b.panel_e, E, n));
-        G_TRY(galois_add(t, x, x1)); ops += 2;
+        // output projection with the residual folded in (narrow for the device: two shares of k and a summing pass)
+        G_TRY(galois_matmul_panel_add(l.wo, b.panel_e, &x, x1, E, n, &b.split_ws)); ops++;
         // feed-forward block: norm -> panel, gate | up in one launch, SwiGLU -> panel, down, residual
         G_TRY(galois_rms_norm_mul_panel(x1, l.ffn_norm, b.panel_e, hp_.rms_eps));
         G_TRY(galois_matmul_panel({{&l.w_gate, &g}, {&l.w_up, &u}}, b.panel_e, E, n));
         G_TRY(galois_silu_mul_panel(g, u, b.panel_f));
-        G_TRY(galois_matmul_panel({{&l.w_down, &t}}, b.panel_f, F, n));
-        G_TRY(galois_add(t, x1, x)); ops += 5;
+        G_TRY(galois_matmul_panel_add(l.w_down, b.panel_f, &x1, x, F, n, &b.split_ws)); ops += 4;
     }
     // the last token's logits, by the decode step's own tail
     {

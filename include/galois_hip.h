@@ -357,6 +357,21 @@ int32_t galois_hip_qkv_attn_decode_f16kv(galois_hip_ctx *ctx, const galois_hip_g
                                          void *v_cache, float *out, int32_t n_head, int32_t head_dim, int32_t n_past,
                                          const int32_t *pos, float freq_scale, float theta_scale, float scale, int32_t head_major_n_ctx);
 
+/* One Q4_0 matrix against the panel with the residual stream added: Y = residual + W . panel (residual may be null),
+ * Y and residual [M][N] f32 -- an output or down projection and the add that follows it (CudaMatMul then add_f32,
+ * src/cuda.rs:1011-1034) as one call.  `workspace` is device memory the call may overwrite (16-byte aligned), or null:
+ *   - with 2 * M * N floats of it, a matrix too narrow to give every compute unit a workgroup (N = 4096 at M = 512:
+ *     86 tiles of 96 columns, or 172 of 48, for 256 CUs) is multiplied as two shares of k by 256 workgroups of 64
+ *     columns, and the pass that adds the residual adds the two partial results as well (M = 512, 11008 -> 4096 with
+ *     the residual: 70 -> 55 us);
+ *   - Y may be the residual itself (the stream updated in place) when the workspace holds M * N floats or more.
+ * The two shapes differ in the order of the f32 sums over k (one chain, or two halves added), i.e. by rounding only;
+ * which one runs depends on shape, workspace and device alone, so a call repeats bit for bit.  One or two launches
+ * (the product, then the adding pass when there is a residual or a second share). */
+int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, const void *W, const void *panel, const float *residual,
+                                              float *Y, int32_t K, int32_t N, int32_t M, void *workspace,
+                                              int64_t workspace_bytes);
+
 /* Causal attention of n_tokens query rows over a KV cache in ONE launch: what a prefill issues per layer as
  * cpy(q -> [D, M, H]), matmul(K^T, q), scale, soft_max under the causal mask, matmul(V, p), cpy(-> [D, H, M])
  * (CudaMatMul src/cuda.rs:867-992, scale and soft_max src/cuda.rs:1597-1663 and 1257-1356, cpy src/cuda.rs:1382-1595),

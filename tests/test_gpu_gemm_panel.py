@@ -78,6 +78,52 @@ def test_matmul_on_the_panel_equals_the_f32_call_bit_for_bit(dev, m, k, ns):
         dev.free(b)
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 4096, 4096), (512, 11008, 4096), (512, 4096, 11008), (130, 256, 200), (300, 768, 1000),
+                                   (17, 512, 4096), (600, 2816, 2048)])
+@pytest.mark.parametrize("with_residual", [True, False])
+def test_matmul_with_the_residual_folded_in_and_in_two_shares_of_k(dev, m, k, n, with_residual):
+    """Y = residual + W . panel.  Without a workspace the call is the plain product and a pass that adds the residual:
+    bit for bit the plain call's result plus the residual.  With a workspace a narrow matrix runs as two shares
+    of k (the first two shapes on 256 CUs) -- another order of the f32 sums, so that result is held to the prefill bar
+    against the oracle, and to 1e-5 of the largest magnitude against the one-launch result; Y may be the residual."""
+    x, (wq,) = _case(m + k + n, m, k, [n])
+    r = np.random.default_rng(n).standard_normal((m, n)).astype(np.float32) if with_residual else None
+    xb, wb = dev.upload(x), dev.upload(wq)
+    pb, _ = _panel(dev, k, m)
+    dev.f32_to_f16_panel(xb, pb, k, m)
+    rb = dev.upload(r) if with_residual else None
+    plain, one, two = dev.alloc(m * n * 4), dev.alloc((m * n + 16) * 4), dev.alloc((m * n + 16) * 4)
+    ws_bytes = 2 * m * n * 4
+    ws = dev.alloc(ws_bytes + 64)
+    for b in (one, two):
+        dev.upload(np.full(m * n + 16, 7.5, np.float32), b)
+    dev.upload(np.full(ws_bytes // 4 + 16, 9.5, np.float32), ws)
+    dev.mul_mat_q4_0_f16_panel([(wb, plain, n)], pb, k, m)
+    dev.mul_mat_q4_0_f16_panel_add(wb, pb, rb, one, k, n, m)
+    dev.mul_mat_q4_0_f16_panel_add(wb, pb, rb, two, k, n, m, ws, ws_bytes)
+    base = dev.download(plain, np.float32, m * n).reshape(m, n)
+    got1, got2 = dev.download(one, np.float32, m * n + 16), dev.download(two, np.float32, m * n + 16)
+    assert np.all(got1[m * n:] == 7.5) and np.all(got2[m * n:] == 7.5), "wrote past the end of Y"
+    assert np.all(dev.download(ws, np.float32, ws_bytes // 4 + 16)[ws_bytes // 4:] == 9.5), "wrote past the end of the workspace"
+    got1, got2 = got1[:m * n].reshape(m, n), got2[:m * n].reshape(m, n)
+    want = base + r if with_residual else base
+    assert np.array_equal(got1.view(np.uint32), want.view(np.uint32))
+    assert np.max(np.abs(got2 - want)) <= 1e-5 * np.max(np.abs(want))
+    cols = np.unique(np.concatenate([[0, n - 1], np.random.default_rng(n).choice(n, min(n, 48), replace=False)]))
+    ref = oracle.mul_mat_q4_0_f32(wq[cols], x)
+    emax, el2 = npref.rel_err(got2[:, cols] - (r[:, cols] if with_residual else 0), ref)
+    assert emax < TOL and el2 < TOL, (emax, el2)
+    if with_residual:   # in place on the residual stream
+        dev.mul_mat_q4_0_f16_panel_add(wb, pb, rb, rb, k, n, m, ws, ws_bytes)
+        assert np.array_equal(dev.download(rb, np.float32, m * n).reshape(m, n).view(np.uint32), got2.view(np.uint32))
+        from galois_amd import GaloisHipError
+        with pytest.raises(GaloisHipError) as ei:      # in place needs somewhere to keep the product
+            dev.mul_mat_q4_0_f16_panel_add(wb, pb, rb, rb, k, n, m)
+        assert ei.value.status == -5
+    for b in [xb, wb, pb, plain, one, two, ws] + ([rb] if with_residual else []):
+        dev.free(b)
+
+
 def _ulps_f16(a, b):
     """Largest distance between two float16 arrays in units of the last place of the larger magnitude."""
     a32, b32 = a.astype(np.float32), b.astype(np.float32)
