@@ -239,10 +239,40 @@ def decode_attention_bench(dev, rng):
     return res
 
 
+def prefill_attention_bench(dev, rng):
+    """Causal attention of 512 rows for 32 heads of 128 in one launch (galois_hip_attn_prefill_*), writing the fp16
+    panel of the output projection: an empty context and a context of 1536 positions, f32 and f16 caches.  The caches
+    rotate over six copies.  flop = the two products under the mask (4 * head_dim per visible (query, key) pair)."""
+    H, D, n = 32, 128, 512
+    E = H * D
+    res = {}
+    q = dev.upload(rng.standard_normal((n, E), dtype=np.float32))
+    panel = dev.alloc(dev.f16_panel_bytes(E, n))
+    for n_past in (0, 1536):
+        L = n_past + n
+        for kv_f16 in (False, True):
+            nbuf = 6 if n_past == 0 else 3
+            host = rng.standard_normal((L, E), dtype=np.float32)
+            host = host.astype(np.float16) if kv_f16 else host
+            kcs = [dev.upload(host) for _ in range(nbuf)]
+            vcs = [dev.upload(host) for _ in range(nbuf)]
+            f = lambda i: dev.attn_prefill(q, kcs[i % nbuf], vcs[i % nbuf], None, panel, H, D, n, n_past, D ** -0.5, kv_f16)
+            us = timed_graph(dev, f, 60, settle_s=SETTLE_S) / 60 * 1e3
+            flop = 4.0 * D * H * sum(n_past + m + 1 for m in range(n))
+            res["n_past_%d_%s_cache" % (n_past, "f16" if kv_f16 else "f32")] = {
+                "us": round(us, 2), "TFLOPs_under_the_mask": round(flop / us / 1e6, 1),
+                "cache_bytes": 2 * L * E * (2 if kv_f16 else 4)}
+            for b_ in kcs + vcs:
+                dev.free(b_)
+    dev.free(q)
+    dev.free(panel)
+    return res
+
+
 SETTLE_STEPS = 150   # decode steps (1.6-3 ms each) run before a plan is timed: the same settling as SETTLE_S
 
 
-def decode_step_bench(dev, reps, with_graph=True):
+def decode_step_bench(dev, reps, with_graph=True, prefill_only=False):
     """BASELINE.json configs[4]: a 32-layer LLaMA-7B-architecture decode step at KV length 2048, issued through the
     host mirror's galois ops, random-init weights quantized on the device.  Returns tokens/s three ways."""
     from galois_amd import host_api as g
@@ -306,21 +336,28 @@ def decode_step_bench(dev, reps, with_graph=True):
         hp = dec.hp
         e, f = hp["n_embd"], hp["n_ff"]
         toks = np.random.default_rng(11).integers(0, hp["n_vocab"], n_tok).astype(np.int32)
+        t_dec = time.time()
         for i, t in enumerate(toks):
             dec.decode(int(t), i, 5)
-        one_by_one = dec.logits().astype(np.float64)
+        one_by_one = dec.logits().astype(np.float64)     # (the download waits for the stream)
+        ms_one_by_one = (time.time() - t_dec) * 1e3
         dec.prefill(toks, 0)
         got = dec.logits().astype(np.float64)
         dec.time_prefill(toks, 0, 4)
         ms = min(dec.time_prefill(toks, 0, 4) for _ in range(3)) / 4
         q4_flop = 2.0 * n_tok * hp["n_layer"] * (4 * e * e + 3 * e * f)
         attn_flop = 2.0 * 2 * n_tok * n_tok * e * hp["n_layer"]     # scores and out over all n_tok keys (the masked half too)
-        return {"tokens": n_tok, "launches": dec.ops_per_prefill(), "ms": round(ms, 3), "tokens_per_s": round(n_tok / ms * 1e3, 0),
-                "q4_0_products_TFLOPs_if_alone": round(q4_flop / ms / 1e9, 1),
+        return {"tokens": n_tok, "library_calls": dec.ops_per_prefill(), "ms": round(ms, 3), "tokens_per_s": round(n_tok / ms * 1e3, 0),
+                "q4_0_flop_over_the_whole_pass_TFLOPs": round(q4_flop / ms / 1e9, 1),
+                "q4_0_flop_over_the_whole_pass_mfma_frac": round(q4_flop / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                 "q4_0_flop": q4_flop, "attention_flop": attn_flop,
-                "speedup_over_decoding_one_by_one": round(n_tok * res["eager_qkv_and_attention_in_one_launch"]["ms_per_token"] / ms, 1),
+                "ms_decoding_one_by_one": round(ms_one_by_one, 1), "speedup_over_decoding_one_by_one": round(ms_one_by_one / ms, 1),
                 "last_logits_vs_one_by_one": cross(got, one_by_one)}
 
+    if prefill_only:
+        res["prefill_512_tokens"] = prefill(dec)
+        dec.close()
+        return res
     for name, fused in (("eager_one_kernel_per_op", 0), ("eager_fused_norm_and_silu", 1), ("eager_grouped_gemv", 2),
                         ("eager_grouped_gemv_fused_attention", 3), ("eager_split_norms", 4),
                         ("eager_qkv_and_attention_in_one_launch", 5)):
@@ -390,6 +427,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip prefill / row-kernel side measurements")
     ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode-step measurement")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="of the 32-layer measurements only the 512-token prefill pass (f32 caches); for runs under the tracer")
     ap.add_argument("--decode-no-graph", action="store_true",
                     help="decode step: eager launches only (graph replays cannot run under the kernel tracer)")
     ap.add_argument("--no-graph", action="store_true",
@@ -535,6 +574,24 @@ def main():
                lambda: dev.mul_mat_q4_0_f16_panel([(w, y, 4096) for w, y in zip(w3, y3)], pb, k, m), 3 * 2.0 * m * k * 4096)
         tpanel("qkv_three_f32_calls_512x4096x4096",
                lambda: [dev.mul_mat_q4_0_f32(w, xp, y, k, 4096, m) for w, y in zip(w3, y3)], 3 * 2.0 * m * k * 4096)
+        # an output / down projection with the residual added: the plain product and the add, against the call that
+        # folds them (with a workspace a narrow matrix runs as two shares of k)
+        kd, nd = 11008, 4096
+        wdn = make_q4_matrix(dev, rng, kd, nd)
+        xd = dev.upload(rng.standard_normal((m, kd), dtype=np.float32))
+        pd = dev.alloc(dev.f16_panel_bytes(kd, m))
+        dev.f32_to_f16_panel(xd, pd, kd, m)
+        res_b, yd, y2d, wsd = dev.upload(rng.standard_normal((m, nd), dtype=np.float32)), dev.alloc(m * nd * 4), dev.alloc(m * nd * 4), dev.alloc(2 * m * nd * 4)
+        tpanel("down_512x11008x4096_then_add",
+               lambda: (dev.mul_mat_q4_0_f16_panel([(wdn, yd, nd)], pd, kd, m), dev.add_f32(yd, res_b, y2d, m * nd, m * nd)), 2.0 * m * kd * nd)
+        tpanel("down_512x11008x4096_with_residual_two_shares_of_k",
+               lambda: dev.mul_mat_q4_0_f16_panel_add(wdn, pd, res_b, y2d, kd, nd, m, wsd, 2 * m * nd * 4), 2.0 * m * kd * nd)
+        tpanel("out_512x4096x4096_then_add",
+               lambda: (dev.mul_mat_q4_0_f16_panel([(w3[0], yd, nd)], pb, k, m), dev.add_f32(yd, res_b, y2d, m * nd, m * nd)), 2.0 * m * k * nd)
+        tpanel("out_512x4096x4096_with_residual_two_shares_of_k",
+               lambda: dev.mul_mat_q4_0_f16_panel_add(w3[0], pb, res_b, y2d, k, nd, m, wsd, 2 * m * nd * 4), 2.0 * m * k * nd)
+        for b_ in (wdn, xd, pd, res_b, yd, y2d, wsd):
+            dev.free(b_)
         extra["prefill_gemm_fp16_panel"] = panel
         for b_ in [pb, gnorm, y2[1]] + w3[1:] + y3:
             dev.free(b_)
@@ -575,6 +632,7 @@ def main():
             v["hbm_frac"] = round(v["GBps"] / HBM_PEAK_GBPS, 4)
         extra["row_kernels"] = rows
         extra["decode_attention"] = decode_attention_bench(dev, rng)
+        extra["prefill_attention"] = prefill_attention_bench(dev, rng)
 
     out = {
         "metric": "Q4_0 GEMV weight GB/s (% of HBM peak); Q4_0 prefill GEMM TFLOP/s @7B shapes",
@@ -594,7 +652,7 @@ def main():
                      "kernel": "gemv_q4_0_group", "bytes_per_launch": avg_bytes, "us_per_launch": round(avg_us, 3)},
     }
     if not args.no_decode:
-        extra["decode_step"] = decode_step_bench(dev, 10, not args.decode_no_graph)
+        extra["decode_step"] = decode_step_bench(dev, 10, not args.decode_no_graph, args.prefill_only)
     if not args.no_cpu:
         weights_host = [dev.download(b, np.uint8, (n, (k // 32) * 18)) for (k, n), b in zip(GEMV_SHAPES, base)]
         res, ncpu = cpu_baseline(weights_host, xs_host, args.cpu_seconds)
