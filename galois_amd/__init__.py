@@ -286,6 +286,18 @@ class Device:
         self._check(self._lib.galois_hip_mul_mat_q4_0_f16_panel_add(self._ctx, _ptr(W), _ptr(panel), _ptr(residual), _ptr(Y), K, N, M,
                                                                     _ptr(workspace), workspace_bytes))
 
+    def mul_mat_q4_0_f16_panel_shares(self, W, panel, shares, shares_bytes, K, N, M):
+        """W . panel as one or two partial results (M * N floats apart) in `shares`; returns how many."""
+        n = C.c_int32(0)
+        self._check(self._lib.galois_hip_mul_mat_q4_0_f16_panel_shares(self._ctx, _ptr(W), _ptr(panel), _ptr(shares), shares_bytes,
+                                                                       K, N, M, C.byref(n)))
+        return n.value
+
+    def add_rms_norm_mul_f16_panel(self, a, b, c, sum_out, weight, panel, ncols, nrows, eps):
+        """sum_out = a (+ b) (+ c); rms_norm(sum_out, eps) * weight into the panel."""
+        self._check(self._lib.galois_hip_add_rms_norm_mul_f16_panel(self._ctx, _ptr(a), _ptr(b), _ptr(c), _ptr(sum_out), _ptr(weight),
+                                                                    _ptr(panel), ncols, nrows, eps))
+
     def attn_prefill(self, q, k_cache, v_cache, out, out_panel, n_head, head_dim, n_tokens, n_past, scale, kv_f16=False):
         """Causal attention of n_tokens rows of q over caches that already hold positions 0 .. n_past + n_tokens - 1;
         the result goes to out (f32) or out_panel (fp16 panel), the other is None."""

@@ -200,12 +200,16 @@ __global__ __launch_bounds__(256) void f32_to_f16_tiles(const float *__restrict_
 // ((x * scale) * weight, rounded to fp16 at the end).  A thread's run is one 16-byte piece of the panel; the sixteen
 // rows of a tile group are given to workgroups of one XCD (blockIdx % 8), so that the pieces of a line meet in
 // one L2 before they are written back.
+// SUM: the row is x + xb + xc first (xb, xc may be null; added in that order, as gemm_sum_pass adds two shares of k
+// and a residual), and that sum is also written to xsum as f32 (xsum may be any of the three inputs: a thread reads
+// its own elements before it writes them) -- the adding pass behind a product and the norm in front of the next one
+// as one launch.
 constexpr int kPanelNormThreads = 512;
-template <int NV>
-__global__ __launch_bounds__(kPanelNormThreads) void rms_norm_to_f16_tiles(const float *__restrict__ x,
-                                                                            const float *__restrict__ w,
+template <int NV, bool SUM = false>
+__global__ __launch_bounds__(kPanelNormThreads) void rms_norm_to_f16_tiles(const float *x, const float *__restrict__ w,
                                                                             _Float16 *__restrict__ y, int M, int K, float eps,
-                                                                            int groups, int groups_per_xcd) {
+                                                                            int groups, int groups_per_xcd, const float *xb = nullptr,
+                                                                            const float *xc = nullptr, float *xsum = nullptr) {
     constexpr int THREADS = kPanelNormThreads;
     __shared__ float part[THREADS / 64];
     const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
@@ -220,9 +224,25 @@ __global__ __launch_bounds__(kPanelNormThreads) void rms_norm_to_f16_tiles(const
     for (int i = 0; i < NV; i++) {
         const int c = threadIdx.x + i * THREADS;
         const bool ok = live && c < nrun;
-        const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)(live ? m : 0) * K) + 2 * (ok ? c : 0);
+        const size_t at = (size_t)(live ? m : 0) * K + 8 * (size_t)(ok ? c : 0);
+        const float4 *src = reinterpret_cast<const float4 *>(x + at);
         v[i][0] = ok ? src[0] : make_float4(0.f, 0.f, 0.f, 0.f);
         v[i][1] = ok ? src[1] : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (SUM) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const float *more = t == 0 ? xb : xc;
+                if (more && ok) {
+                    const float4 p = reinterpret_cast<const float4 *>(more + at)[0], q = reinterpret_cast<const float4 *>(more + at)[1];
+                    v[i][0] = make_float4(v[i][0].x + p.x, v[i][0].y + p.y, v[i][0].z + p.z, v[i][0].w + p.w);
+                    v[i][1] = make_float4(v[i][1].x + q.x, v[i][1].y + q.y, v[i][1].z + q.z, v[i][1].w + q.w);
+                }
+            }
+            if (ok) {
+                __builtin_nontemporal_store(float4_t{v[i][0].x, v[i][0].y, v[i][0].z, v[i][0].w}, reinterpret_cast<float4_t *>(xsum + at));
+                __builtin_nontemporal_store(float4_t{v[i][1].x, v[i][1].y, v[i][1].z, v[i][1].w}, reinterpret_cast<float4_t *>(xsum + at) + 1);
+            }
+        }
     }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
@@ -850,6 +870,34 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel(galois_hip_ctx *ctx, const 
     GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel launch");
 }
 
+namespace {
+
+// Whether one matrix against the panel is better multiplied as two shares of k, each a workgroup of 64 columns, than
+// as whole-k tiles: the cost model of gemm_launch_any (rounds of workgroups x cost of a stage x stages; a 64-column
+// stage on a full device at 0.75 of a 96-column one) plus the pass that adds the two partial results, which costs
+// about fourteen stages per 2^21 results.  Measured at M = 512 on 256 CUs: 11008 -> 4096 70.3 -> 54.8 us,
+// 4096 -> 4096 32.5 -> 30.2 us (both with the residual); the shapes the model leaves whole are slower when forced
+// into shares.
+bool gemm_two_shares_pay(const galois_hip_ctx *ctx, int K, int N, int M) {
+    const int64_t m_tiles = (M + GM - 1) / GM, cus = ctx->n_cu > 0 ? ctx->n_cu : 256, stages = K / 64;
+    const int64_t wg96 = ((int64_t)N + 95) / 96 * m_tiles, wg48 = ((int64_t)N + 47) / 48 * m_tiles, wg64x2 = ((int64_t)N + 63) / 64 * m_tiles * 2;
+    const int64_t mn = (int64_t)M * N;
+    const double c96 = (double)((wg96 + cus - 1) / cus) * stages, c48 = 0.65 * (double)((wg48 + cus - 1) / cus) * stages;
+    const double c64x2 = 0.75 * (double)((wg64x2 + cus - 1) / cus) * (stages / 2 + 2) + 14.0 * (double)mn / (double)(1 << 21);
+    return K >= 512 && mn % 4 == 0 && c64x2 < c96 && c64x2 < c48;
+}
+
+// W . panel into dst as one result (shares = 1) or as two partial results M * N floats apart (shares = 2).
+int32_t gemm_launch_shares(galois_hip_ctx *ctx, const void *W, const _Float16 *panel, float *dst, int K, int N, int M, int shares) {
+    gemm_mats mats = {};
+    mats.W[0] = (const uint8_t *)W, mats.Y[0] = dst, mats.N[0] = N;
+    if (shares == 1) return gemm_launch_any(ctx, mats, 1, panel, K, M);
+    gemm_concat(mats, 1);
+    return gemm_launch<64>(ctx, mats, panel, K, M, 2, (size_t)M * N);
+}
+
+}  // namespace
+
 // One matrix against the panel with a residual added, and the k-split shape for matrices too narrow to fill the device.
 extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, const void *W, const void *panel, const float *residual,
                                                          float *Y, int32_t K, int32_t N, int32_t M, void *workspace,
@@ -862,24 +910,10 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, co
                GALOIS_HIP_E_ALIGN, "mul_mat_q4_0_f16_panel_add: 16-byte aligned operands");
     GH_REQUIRE(ctx, workspace_bytes >= 0, GALOIS_HIP_E_SHAPE, "mul_mat_q4_0_f16_panel_add: workspace_bytes");
     GH_BIND(ctx);
-    gemm_mats mats = {};
-    mats.W[0] = (const uint8_t *)W, mats.Y[0] = Y, mats.N[0] = N;
-    // Two shares of k, each a workgroup of 64 columns, when that fills the device better than whole-k tiles do: the
-    // cost model of gemm_launch_any (rounds of workgroups x cost of a stage x stages; a 64-column stage on a full
-    // device at 0.75 of a 96-column one) plus the pass that adds the two partial results, which costs about fourteen
-    // stages per 2^21 results.  Measured at M = 512 on 256 CUs: 11008 -> 4096 70.3 -> 54.8 us, 4096 -> 4096 32.5 -> 30.2 us
-    // (both with the residual), and the shapes the model leaves whole are slower when forced into shares.
-    const int64_t m_tiles = (M + GM - 1) / GM, cus = ctx->n_cu > 0 ? ctx->n_cu : 256, stages = K / 64;
-    const int64_t wg96 = ((int64_t)N + 95) / 96 * m_tiles, wg48 = ((int64_t)N + 47) / 48 * m_tiles, wg64x2 = ((int64_t)N + 63) / 64 * m_tiles * 2;
     const int64_t mn = (int64_t)M * N;
-    const double c96 = (double)((wg96 + cus - 1) / cus) * stages, c48 = 0.65 * (double)((wg48 + cus - 1) / cus) * stages;
-    const double c64x2 = 0.75 * (double)((wg64x2 + cus - 1) / cus) * (stages / 2 + 2) + 14.0 * (double)mn / (double)(1 << 21);
-    const bool can_split = workspace && workspace_bytes >= 2 * mn * (int64_t)sizeof(float) && K >= 512 && mn % 4 == 0;
     const dim3 sum_grid((unsigned)((mn / 4 + 255) / 256));
-    if (can_split && c64x2 < c96 && c64x2 < c48) {
-        mats.Y[0] = static_cast<float *>(workspace);
-        gemm_concat(mats, 1);
-        const int32_t st = gemm_launch<64>(ctx, mats, (const _Float16 *)panel, K, M, 2, (size_t)mn);
+    if (gemm_two_shares_pay(ctx, K, N, M) && workspace && workspace_bytes >= 2 * mn * (int64_t)sizeof(float)) {
+        const int32_t st = gemm_launch_shares(ctx, W, (const _Float16 *)panel, static_cast<float *>(workspace), K, N, M, 2);
         if (st != GALOIS_HIP_OK) return st;
         hipLaunchKernelGGL(gemm_sum_pass, sum_grid, dim3(256), 0, ctx->stream, static_cast<const float4 *>(workspace),
                            reinterpret_cast<const float4 *>(residual), reinterpret_cast<float4 *>(Y), mn / 4, mn / 4);
@@ -891,8 +925,7 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, co
                        "mul_mat_q4_0_f16_panel_add: Y may be the residual only with a workspace of M * N floats or more");
             prod = static_cast<float *>(workspace);
         }
-        mats.Y[0] = prod;
-        const int32_t st = gemm_launch_any(ctx, mats, 1, (const _Float16 *)panel, K, M);
+        const int32_t st = gemm_launch_shares(ctx, W, (const _Float16 *)panel, prod, K, N, M, 1);
         if (st != GALOIS_HIP_OK) return st;
         if (residual) {
             if (mn % 4 == 0)
@@ -903,4 +936,50 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, co
         }
     }
     GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel_add launch");
+}
+
+// The product alone, as the shares it is computed in: what galois_hip_mul_mat_q4_0_f16_panel_add does before its adding
+// pass, for callers whose next op can do the adding (galois_hip_add_rms_norm_mul_f16_panel).
+extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_shares(galois_hip_ctx *ctx, const void *W, const void *panel, float *shares,
+                                                            int64_t shares_bytes, int32_t K, int32_t N, int32_t M, int32_t *n_shares) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, W && panel && shares && n_shares, GALOIS_HIP_E_NULL, "mul_mat_q4_0_f16_panel_shares");
+    *n_shares = 0;
+    GH_REQUIRE(ctx, gemm_panel_shape_ok(K, M) && N > 0 && (int64_t)M * N < ((int64_t)1 << 31), GALOIS_HIP_E_SHAPE,
+               "mul_mat_q4_0_f16_panel_shares: K a positive multiple of 256, (M + 16) * K below 2^31, N positive, M * N below 2^31");
+    GH_REQUIRE(ctx, gh_aligned(W, 16) && gh_aligned(panel, 16) && gh_aligned(shares, 16), GALOIS_HIP_E_ALIGN,
+               "mul_mat_q4_0_f16_panel_shares: 16-byte aligned operands");
+    const int64_t mn = (int64_t)M * N;
+    GH_REQUIRE(ctx, shares_bytes >= mn * (int64_t)sizeof(float), GALOIS_HIP_E_SHAPE,
+               "mul_mat_q4_0_f16_panel_shares: room for at least one result of M * N floats");
+    GH_BIND(ctx);
+    const int n = gemm_two_shares_pay(ctx, K, N, M) && shares_bytes >= 2 * mn * (int64_t)sizeof(float) ? 2 : 1;
+    const int32_t st = gemm_launch_shares(ctx, W, (const _Float16 *)panel, shares, K, N, M, n);
+    if (st != GALOIS_HIP_OK) return st;
+    *n_shares = n;
+    GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel_shares launch");
+}
+
+// sum_out = a (+ b) (+ c), and rms_norm(sum_out, eps) * weight into the panel, one launch.
+extern "C" int32_t galois_hip_add_rms_norm_mul_f16_panel(galois_hip_ctx *ctx, const float *a, const float *b, const float *c,
+                                                         float *sum_out, const float *weight, void *panel, int32_t ncols,
+                                                         int32_t nrows, float eps) {
+    const int32_t st = panel_args(ctx, a, weight, panel, ncols, nrows, "add_rms_norm_mul_f16_panel");
+    if (st != GALOIS_HIP_OK) return st;
+    GH_REQUIRE(ctx, sum_out, GALOIS_HIP_E_NULL, "add_rms_norm_mul_f16_panel: sum_out");
+    GH_REQUIRE(ctx, gh_aligned(b, 16) && gh_aligned(c, 16) && gh_aligned(sum_out, 16), GALOIS_HIP_E_ALIGN,
+               "add_rms_norm_mul_f16_panel: 16-byte aligned operands");
+    const int nv = (ncols / 8 + kPanelNormThreads - 1) / kPanelNormThreads;
+    GH_REQUIRE(ctx, nv <= 4, GALOIS_HIP_E_SHAPE, "add_rms_norm_mul_f16_panel: rows of at most 16384 columns");
+    GH_BIND(ctx);
+    const int groups = (nrows + 15) / 16, per_xcd = (groups + 7) / 8;
+    const dim3 grid((unsigned)(8 * per_xcd * 16)), block(kPanelNormThreads);
+    _Float16 *y = (_Float16 *)panel;
+    if (nv <= 1)
+        hipLaunchKernelGGL((rms_norm_to_f16_tiles<1, true>), grid, block, 0, ctx->stream, a, weight, y, nrows, ncols, eps, groups, per_xcd, b, c, sum_out);
+    else if (nv <= 2)
+        hipLaunchKernelGGL((rms_norm_to_f16_tiles<2, true>), grid, block, 0, ctx->stream, a, weight, y, nrows, ncols, eps, groups, per_xcd, b, c, sum_out);
+    else
+        hipLaunchKernelGGL((rms_norm_to_f16_tiles<4, true>), grid, block, 0, ctx->stream, a, weight, y, nrows, ncols, eps, groups, per_xcd, b, c, sum_out);
+    GH_LAUNCH_CHECK(ctx, "add_rms_norm_mul_f16_panel launch");
 }

@@ -133,6 +133,15 @@ GResult galois_matmul_panel_add(const Tensor &w, const Tensor &panel, const Tens
 GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                            Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale);
 
+// The product alone as its one or two shares of k (galois_hip_mul_mat_q4_0_f16_panel_shares): shares is an F32 tensor of
+// at least N * M elements (2 * N * M let a narrow matrix run as two shares); *n_shares says how many partial results
+// it now holds, N * M elements apart.
+GResult galois_matmul_panel_shares(const Tensor &w, const Tensor &panel, Tensor &shares, size_t K, size_t M, int32_t *n_shares);
+// sum_out = the n_shares partial results in `shares` + residual (may be null), and rms_norm(sum_out, eps) * weight into
+// the panel, in one launch (galois_hip_add_rms_norm_mul_f16_panel).  sum_out: F32 [ncols, nrows]; it may be residual.
+GResult galois_add_rms_norm_mul_panel(const Tensor &shares, int32_t n_shares, const Tensor *residual, Tensor &sum_out,
+                                      const Tensor &weight, Tensor &panel, float eps);
+
 // Causal attention of all rows of q ([n_embd, n] f32, rotated) over caches ([n_embd, n_ctx], both f32 or both f16) that
 // already hold positions 0 .. n_past + n - 1, in one launch (galois_hip_attn_prefill_f32 / _f16kv; heads of 128).
 // dst is either an F32 tensor [n_embd, n] or an F16 panel of galois_panel_elems(n_embd, n) elements.

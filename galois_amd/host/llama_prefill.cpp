@@ -109,6 +109,44 @@ GResult galois_matmul_panel_add(const Tensor &w, const Tensor &panel, const Tens
         workspace ? (int64_t)(workspace->dim().elem_count() * sizeof(float)) : 0));
 }
 
+GResult galois_matmul_panel_shares(const Tensor &w, const Tensor &panel, Tensor &shares, size_t K, size_t M, int32_t *n_shares) {
+    if (!n_shares) return err(GError::Unexpected, "galois_matmul_panel_shares: n_shares is required");
+    if (!panel.device().is_gpu() || panel.dtype() != GGmlType::F16 || panel.dim().elem_count() < galois_panel_elems(K, M))
+        return err(GError::ShapeError, "galois_matmul_panel_shares: an F16 Gpu panel of galois_panel_elems(K, M) elements");
+    const auto &dev = panel.device().gpu;
+    if (!w.device().is_gpu() || w.device().gpu != dev || !shares.device().is_gpu() || shares.device().gpu != dev)
+        return err(GError::Unimplemented, "galois_matmul_panel_shares: Gpu tensors on the panel's device");
+    if (w.dtype() != GGmlType::Q4_0 || shares.dtype() != GGmlType::F32 || !w.dim().ggml_is_contiguous(w.dtype()) ||
+        !shares.dim().ggml_is_contiguous(shares.dtype()))
+        return err(GError::Unimplemented, "galois_matmul_panel_shares: a contiguous Q4_0 matrix and an F32 tensor for the shares");
+    const size_t N = w.dim().shape[1];
+    if (w.dim().shape[0] != K || w.dim().elem_count() != K * N || shares.dim().elem_count() < N * M)
+        return err(GError::ShapeError, "galois_matmul_panel_shares: w [K, N], shares of at least N * M elements");
+    return dev->check(galois_hip_mul_mat_q4_0_f16_panel_shares(dev->ctx(), w.data(), panel.data(), (float *)shares.data(),
+                                                               (int64_t)(shares.dim().elem_count() * sizeof(float)), (int32_t)K,
+                                                               (int32_t)N, (int32_t)M, n_shares));
+}
+
+GResult galois_add_rms_norm_mul_panel(const Tensor &shares, int32_t n_shares, const Tensor *residual, Tensor &sum_out,
+                                      const Tensor &weight, Tensor &panel, float eps) {
+    std::shared_ptr<CudaDevice> dev;
+    size_t K, M;
+    G_TRY(panel_operands(sum_out, panel, &dev, &K, &M, "galois_add_rms_norm_mul_panel"));
+    if (n_shares < 1 || n_shares > 2) return err(GError::ShapeError, "galois_add_rms_norm_mul_panel: one or two shares");
+    if (!shares.device().is_gpu() || shares.device().gpu != dev || shares.dtype() != GGmlType::F32 ||
+        !shares.dim().ggml_is_contiguous(shares.dtype()) || shares.dim().elem_count() < (size_t)n_shares * K * M)
+        return err(GError::ShapeError, "galois_add_rms_norm_mul_panel: shares F32 on the Gpu, n_shares results of sum_out's size");
+    if (residual && (!residual->device().is_gpu() || residual->device().gpu != dev || residual->dtype() != GGmlType::F32 ||
+                     !residual->dim().ggml_is_contiguous(residual->dtype()) || residual->dim().elem_count() != K * M))
+        return err(GError::ShapeError, "galois_add_rms_norm_mul_panel: residual F32 of sum_out's shape");
+    if (!weight.device().is_gpu() || weight.dtype() != GGmlType::F32 || weight.dim().elem_count() != K)
+        return err(GError::ShapeError, "galois_add_rms_norm_mul_panel: weight must be ne00 F32 elements on the Gpu");
+    const float *a = (const float *)shares.data();
+    return dev->check(galois_hip_add_rms_norm_mul_f16_panel(dev->ctx(), a, n_shares == 2 ? a + K * M : nullptr,
+                                                            residual ? (const float *)residual->data() : nullptr, (float *)sum_out.data(),
+                                                            (const float *)weight.data(), panel.data(), (int32_t)K, (int32_t)M, eps));
+}
+
 GResult galois_attn_prefill(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &dst, size_t n_head,
                             int32_t n_past, float scale) {
     for (const Tensor *t : {&q, &k_cache, &v_cache, (const Tensor *)&dst})
@@ -147,8 +185,9 @@ static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t 
 }
 
 GResult LlamaDecoder::prefill_buffers(size_t n, size_t keys) {
-    if (n <= pf_.rows && keys <= pf_.keys) return GError{};
     const size_t E = hp_.n_embd, F = hp_.n_ff, H = hp_.n_head, D = E / H;
+    const bool op_sequence = D != 128;  // the attention as single ops needs the scores and the permuted copies
+    if (n <= pf_.rows && (keys <= pf_.keys || !op_sequence)) return GError{};
     const size_t rows = n > pf_.rows ? n : pf_.rows, kk = keys > pf_.keys ? keys : pf_.keys;
     Prefill b;  // the old buffers are released when b replaces them: nothing of an earlier call is still queued on them
                 // only once the stream has drained
@@ -156,13 +195,16 @@ GResult LlamaDecoder::prefill_buffers(size_t n, size_t keys) {
     const GGmlType F32 = GGmlType::F32;
     G_TRY(mk(&b.tok, GGmlType::I32, dev_, rows));
     G_TRY(mk(&b.pos, GGmlType::I32, dev_, rows));
-    for (Tensor *t : {&b.x, &b.x1, &b.q, &b.k, &b.v, &b.ao}) G_TRY(mk(t, F32, dev_, E, rows));
+    for (Tensor *t : {&b.x, &b.x1, &b.q, &b.k, &b.v}) G_TRY(mk(t, F32, dev_, E, rows));
     G_TRY(mk(&b.qr, F32, dev_, D, H, rows));
     G_TRY(mk(&b.kr, F32, dev_, D, H, rows));
-    G_TRY(mk(&b.q3, F32, dev_, D, rows, H));
-    G_TRY(mk(&b.o, F32, dev_, D, rows, H));
-    G_TRY(mk(&b.s, F32, dev_, kk, rows, H));
-    G_TRY(mk(&b.p, F32, dev_, kk, rows, H));
+    if (op_sequence) {
+        G_TRY(mk(&b.ao, F32, dev_, E, rows));
+        G_TRY(mk(&b.q3, F32, dev_, D, rows, H));
+        G_TRY(mk(&b.o, F32, dev_, D, rows, H));
+        G_TRY(mk(&b.s, F32, dev_, kk, rows, H));
+        G_TRY(mk(&b.p, F32, dev_, kk, rows, H));
+    }
     G_TRY(mk(&b.g, F32, dev_, F, rows));
     G_TRY(mk(&b.u, F32, dev_, F, rows));
     G_TRY(mk(&b.panel_e, GGmlType::F16, dev_, galois_panel_elems(E, rows)));
@@ -193,14 +235,17 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
         G_TRY(b.tok.view(0, 1, one, &tok));
         G_TRY(b.pos.view(0, 1, one, &pos));
         for (auto pr : {std::make_pair(&b.x, &x), std::make_pair(&b.x1, &x1), std::make_pair(&b.q, &q),
-                        std::make_pair(&b.k, &k), std::make_pair(&b.v, &v), std::make_pair(&b.ao, &ao)})
+                        std::make_pair(&b.k, &k), std::make_pair(&b.v, &v)})
             G_TRY(pr.first->view(0, 2, en, pr.second));
         G_TRY(b.qr.view(0, 3, dhn, &qr));
         G_TRY(b.kr.view(0, 3, dhn, &kr));
-        G_TRY(b.q3.view(0, 3, dnh, &q3));
-        G_TRY(b.o.view(0, 3, dnh, &o));
-        G_TRY(b.s.view(0, 3, lnh, &s));
-        G_TRY(b.p.view(0, 3, lnh, &p));
+        if (D != 128) {
+            G_TRY(b.ao.view(0, 2, en, &ao));
+            G_TRY(b.q3.view(0, 3, dnh, &q3));
+            G_TRY(b.o.view(0, 3, dnh, &o));
+            G_TRY(b.s.view(0, 3, lnh, &s));
+            G_TRY(b.p.view(0, 3, lnh, &p));
+        }
         G_TRY(b.g.view(0, 2, fn, &g));
         G_TRY(b.u.view(0, 2, fn, &u));
     }
@@ -216,9 +261,11 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
     const bool one_launch = D == 128;  // the attention of a layer as one launch (galois_attn_prefill)
     const float attn_scale = 1.0f / sqrtf((float)D);
     G_TRY(galois_get_rows(tok_embd_, tok, x)); ops++;
-    for (Layer &l : layers_) {
-        // attention block: norm -> panel, q | k | v in one launch
-        G_TRY(galois_rms_norm_mul_panel(x, l.attn_norm, b.panel_e, hp_.rms_eps));
+    // the first layer's attention norm; every later one rides on the pass that adds the down projection's shares
+    G_TRY(galois_rms_norm_mul_panel(x, layers_[0].attn_norm, b.panel_e, hp_.rms_eps)); ops++;
+    for (size_t li = 0; li < layers_.size(); li++) {
+        Layer &l = layers_[li];
+        // attention block: (norm -> panel, above or at the end of the layer before) q | k | v in one launch
         Tensor q_heads, k_heads;
         {
             const size_t dhn[3] = {D, H, n};
@@ -234,11 +281,11 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
             Tensor kr_cache;
             const size_t dhn[3] = {D, H, n};
             G_TRY(k_rows.view(0, 3, dhn, &kr_cache));
-            G_TRY(galois_matmul_panel({{&l.wq, &q}, {&l.wk, &k}, {&l.wv, &v_rows}}, b.panel_e, E, n)); ops += 2;
+            G_TRY(galois_matmul_panel({{&l.wq, &q}, {&l.wk, &k}, {&l.wv, &v_rows}}, b.panel_e, E, n)); ops++;
             G_TRY(galois_rope_custom(rope, q_heads, pos, qr));
             G_TRY(galois_rope_custom(rope, k_heads, pos, kr_cache)); ops += 2;
         } else {
-            G_TRY(galois_matmul_panel({{&l.wq, &q}, {&l.wk, &k}, {&l.wv, &v}}, b.panel_e, E, n)); ops += 2;
+            G_TRY(galois_matmul_panel({{&l.wq, &q}, {&l.wk, &k}, {&l.wv, &v}}, b.panel_e, E, n)); ops++;
             G_TRY(galois_rope_custom(rope, q_heads, pos, qr));
             G_TRY(galois_rope_custom(rope, k_heads, pos, kr)); ops += 2;
             Tensor kr_flat;
@@ -279,13 +326,21 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
             }
             G_TRY(galois_to_panel(ao, b.panel_e)); ops++;
         }
-        // output projection with the residual folded in (narrow for the device: two shares of k and a summing pass)
-        G_TRY(galois_matmul_panel_add(l.wo, b.panel_e, &x, x1, E, n, &b.split_ws)); ops++;
-        // feed-forward block: norm -> panel, gate | up in one launch, SwiGLU -> panel, down, residual
-        G_TRY(galois_rms_norm_mul_panel(x1, l.ffn_norm, b.panel_e, hp_.rms_eps));
+        // output projection as its shares of k (narrow for the device: two); the pass that adds them and the residual
+        // stream also writes the feed-forward norm's panel
+        int32_t shares = 0;
+        G_TRY(galois_matmul_panel_shares(l.wo, b.panel_e, b.split_ws, E, n, &shares));
+        G_TRY(galois_add_rms_norm_mul_panel(b.split_ws, shares, &x, x1, l.ffn_norm, b.panel_e, hp_.rms_eps)); ops += 2;
+        // feed-forward block: gate | up in one launch, SwiGLU -> panel, down as shares; the adding pass writes the next
+        // layer's attention norm (after the last layer there is no next norm: the plain adding pass)
         G_TRY(galois_matmul_panel({{&l.w_gate, &g}, {&l.w_up, &u}}, b.panel_e, E, n));
-        G_TRY(galois_silu_mul_panel(g, u, b.panel_f));
-        G_TRY(galois_matmul_panel_add(l.w_down, b.panel_f, &x1, x, F, n, &b.split_ws)); ops += 4;
+        G_TRY(galois_silu_mul_panel(g, u, b.panel_f)); ops += 2;
+        if (li + 1 < layers_.size()) {
+            G_TRY(galois_matmul_panel_shares(l.w_down, b.panel_f, b.split_ws, F, n, &shares));
+            G_TRY(galois_add_rms_norm_mul_panel(b.split_ws, shares, &x1, x, layers_[li + 1].attn_norm, b.panel_e, hp_.rms_eps)); ops += 2;
+        } else {
+            G_TRY(galois_matmul_panel_add(l.w_down, b.panel_f, &x1, x, F, n, &b.split_ws)); ops++;
+        }
     }
     // the last token's logits, by the decode step's own tail
     {

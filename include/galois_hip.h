@@ -372,6 +372,21 @@ int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, const void *W
                                               float *Y, int32_t K, int32_t N, int32_t M, void *workspace,
                                               int64_t workspace_bytes);
 
+/* The product of galois_hip_mul_mat_q4_0_f16_panel_add alone, as the shares of k it is computed in, for a caller whose
+ * next op does the adding (galois_hip_add_rms_norm_mul_f16_panel below): *n_shares = 1 or 2 partial results [M][N] f32
+ * at shares and shares + M * N, whose sum (in that order) is W . panel.  Two only when that pays for the shape
+ * and shares_bytes holds 2 * M * N floats; shares_bytes must hold M * N. */
+int32_t galois_hip_mul_mat_q4_0_f16_panel_shares(galois_hip_ctx *ctx, const void *W, const void *panel, float *shares,
+                                                 int64_t shares_bytes, int32_t K, int32_t N, int32_t M, int32_t *n_shares);
+
+/* sum_out = a (+ b) (+ c) (b, c may be null; added in that order), all [nrows][ncols] f32, and
+ * rms_norm(sum_out, eps) * weight into the fp16 panel (as galois_hip_rms_norm_mul_f16_panel would write it from
+ * sum_out): the adding pass behind an output / down projection (its one or two shares and the residual stream) and
+ * the norm in front of the next product as one launch (add_f32 + rms_norm_f32 + mul_f32 of the reference,
+ * src/cuda.rs:1146-1215).  sum_out may be one of a, b, c. */
+int32_t galois_hip_add_rms_norm_mul_f16_panel(galois_hip_ctx *ctx, const float *a, const float *b, const float *c, float *sum_out,
+                                              const float *weight, void *panel, int32_t ncols, int32_t nrows, float eps);
+
 /* Causal attention of n_tokens query rows over a KV cache in ONE launch: what a prefill issues per layer as
  * cpy(q -> [D, M, H]), matmul(K^T, q), scale, soft_max under the causal mask, matmul(V, p), cpy(-> [D, H, M])
  * (CudaMatMul src/cuda.rs:867-992, scale and soft_max src/cuda.rs:1597-1663 and 1257-1356, cpy src/cuda.rs:1382-1595),

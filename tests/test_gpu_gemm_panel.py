@@ -124,6 +124,43 @@ def test_matmul_with_the_residual_folded_in_and_in_two_shares_of_k(dev, m, k, n,
         dev.free(b)
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 11008, 4096), (512, 4096, 4096), (130, 256, 512), (33, 768, 2048)])
+@pytest.mark.parametrize("with_residual", [True, False])
+def test_shares_then_adding_pass_fused_with_the_next_norm(dev, m, k, n, with_residual):
+    """The product left as its shares of k, then one launch that adds them (and the residual) and writes the next
+    norm's panel: the sum and the panel equal, bit for bit, those of the folded matmul followed by the norm-to-panel
+    call (the same additions in the same order, the same norm arithmetic)."""
+    x, (wq,) = _case(m + k + n + 1, m, k, [n])
+    rng = np.random.default_rng(n + m)
+    r = rng.standard_normal((m, n)).astype(np.float32) if with_residual else None
+    g = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    xb, wb, gb = dev.upload(x), dev.upload(wq), dev.upload(g)
+    rb = dev.upload(r) if with_residual else None
+    pb, _ = _panel(dev, k, m)
+    dev.f32_to_f16_panel(xb, pb, k, m)
+    ws_bytes = 2 * m * n * 4
+    ws, y_ref, y_got = dev.alloc(ws_bytes), dev.alloc(m * n * 4), dev.alloc(m * n * 4)
+    p_ref, nb = _panel(dev, n, m)
+    p_got, _ = _panel(dev, n, m)
+    dev.mul_mat_q4_0_f16_panel_add(wb, pb, rb, y_ref, k, n, m, ws, ws_bytes)
+    dev.rms_norm_mul_f16_panel(y_ref, gb, p_ref, n, m, 1e-6)
+    shares = dev.mul_mat_q4_0_f16_panel_shares(wb, pb, ws, ws_bytes, k, n, m)
+    assert shares in (1, 2)
+    if m == 512 and dev.info()["n_cu"] == 256:
+        assert shares == 2      # 4096 columns at 512 rows leave CUs idle as whole-k tiles
+    dev.add_rms_norm_mul_f16_panel(ws, ws.view(m * n * 4) if shares == 2 else None, rb, y_got, gb, p_got, n, m, 1e-6)
+    assert np.array_equal(dev.download(y_got, np.uint32, m * n), dev.download(y_ref, np.uint32, m * n))
+    assert np.array_equal(dev.download(p_got, np.uint8, nb), dev.download(p_ref, np.uint8, nb))
+    # with room for one result only the product comes whole
+    assert dev.mul_mat_q4_0_f16_panel_shares(wb, pb, ws, m * n * 4, k, n, m) == 1
+    if with_residual:   # the sum may replace the residual in place
+        dev.add_rms_norm_mul_f16_panel(ws, None, rb, rb, gb, p_got, n, m, 1e-6)
+        whole = dev.download(ws, np.float32, m * n)
+        assert np.array_equal(dev.download(rb, np.float32, m * n), whole + r.reshape(-1))
+    for b in [xb, wb, gb, pb, ws, y_ref, y_got, p_ref, p_got] + ([rb] if with_residual else []):
+        dev.free(b)
+
+
 def _ulps_f16(a, b):
     """Largest distance between two float16 arrays in units of the last place of the larger magnitude."""
     a32, b32 = a.astype(np.float32), b.astype(np.float32)
