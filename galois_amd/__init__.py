@@ -286,6 +286,11 @@ class Device:
         self._check(self._lib.galois_hip_mul_mat_q4_0_f16_panel_add(self._ctx, _ptr(W), _ptr(panel), _ptr(residual), _ptr(Y), K, N, M,
                                                                     _ptr(workspace), workspace_bytes))
 
+    def mul_mat_q4_0_swiglu_f16_panel(self, W_gate, W_up, panel, panel_out, K, N, M):
+        """panel_out = the panel of silu(W_gate . x) * (W_up . x) for x given as `panel`, one launch."""
+        self._check(self._lib.galois_hip_mul_mat_q4_0_swiglu_f16_panel(self._ctx, _ptr(W_gate), _ptr(W_up), _ptr(panel), _ptr(panel_out),
+                                                                       K, N, M))
+
     def mul_mat_q4_0_f16_panel_shares(self, W, panel, shares, shares_bytes, K, N, M):
         """W . panel as one or two partial results (M * N floats apart) in `shares`; returns how many."""
         n = C.c_int32(0)

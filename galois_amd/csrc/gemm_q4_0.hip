@@ -321,10 +321,20 @@ struct gemm_mats {
     int32_t N[GEMM_MAX_MATS];
     int32_t col0[GEMM_MAX_MATS];  // first concatenated column of each matrix; unused entries hold INT_MAX
     int32_t n_total;              // columns of the concatenation
+    // SwiGLU pairing (96-column tiles only): W[0] = gate, W[1] = up, both N[0] rows.  Tile t holds rows 48 t .. 48 t + 47
+    // of the gate matrix in its first 48 columns and the same rows of the up matrix in its last 48, so a consumer wave
+    // has both products of an element in its registers and stores silu(gate) * up, as fp16, into the panel of the
+    // [N[0], M] operand at swiglu_out.  n_total = 96 * ceil(N[0] / 48) then.
+    _Float16 *swiglu_out;
 };
 
 // Row `c` of the concatenated weights (clamped to the last one): its bytes.
 __device__ __forceinline__ const uint8_t *gemm_w_row(const gemm_mats &mats, int c, size_t wrow_bytes) {
+    if (mats.swiglu_out) {
+        const int t = c / 96, sub = c - t * 96, up = sub >= 48;
+        const int r = min(t * 48 + sub - 48 * up, mats.N[0] - 1);
+        return mats.W[up] + (size_t)r * wrow_bytes;
+    }
     c = min(c, mats.n_total - 1);
     const uint8_t *W = mats.W[0];
     int first = 0;
@@ -617,8 +627,32 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
         GEMM_DRAIN_A(a3);
     }
 
-    // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e.  A lane's column lies in one of the
-    // matrices of the launch: the result goes to that matrix's Y.
+    // C layout of the 16x16 MFMA: column = lane % 16, row = 4 * (lane / 16) + e.
+    if (NF == 6 && mats.swiglu_out) {
+        // columns j and j + 3 of the wave's tile are the gate and the up product of one output column: silu(gate) * up
+        // (silu_f32 then mul_f32, unary.cu:1-10, mul.cu:3-12, with the arithmetic of f32_to_f16_tiles<true>) goes
+        // to the panel as fp16: element (m, n) lies in tile (m / 16, n / 32) of 1 KB, 16-byte piece ((n % 32) / 8) * 16
+        // + m % 16, at n % 8.  Rows of the panel past M were zeros in the input panel, so their products are zeros.
+        const int N = mats.N[0], m_pad = (M + 15) & ~15;
+        unsigned char *out = reinterpret_cast<unsigned char *>(mats.swiglu_out);
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const int n = (n0 / 96) * 48 + j * 16 + (lane & 15);
+            const size_t col_at = (size_t)(n >> 5) * 1024 + (size_t)((n & 31) >> 3) * 256 + (size_t)(n & 7) * 2;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + e;
+                    const float g = acc[i][j][e], u = acc[i][j + 3 < NF ? j + 3 : j][e];
+                    const _Float16 h = (_Float16)(g / (1.0f + expf(-g)) * u);
+                    if (m < m_pad && n < N)
+                        *reinterpret_cast<_Float16 *>(out + (size_t)(m >> 4) * (size_t)(N >> 5) * 1024 + col_at + (size_t)(m & 15) * 16) = h;
+                }
+        }
+        return;
+    }
+    // A lane's column lies in one of the matrices of the launch: the result goes to that matrix's Y.
 #pragma unroll
     for (int j = 0; j < NF; j++) {
         const int n = n0 + ncol0 + j * 16 + (lane & 15);
@@ -982,4 +1016,25 @@ extern "C" int32_t galois_hip_add_rms_norm_mul_f16_panel(galois_hip_ctx *ctx, co
     else
         hipLaunchKernelGGL((rms_norm_to_f16_tiles<4, true>), grid, block, 0, ctx->stream, a, weight, y, nrows, ncols, eps, groups, per_xcd, b, c, sum_out);
     GH_LAUNCH_CHECK(ctx, "add_rms_norm_mul_f16_panel launch");
+}
+
+// gate | up and the SwiGLU between them and the down projection in one launch: the panel of silu(Wg . x) * (Wu . x).
+extern "C" int32_t galois_hip_mul_mat_q4_0_swiglu_f16_panel(galois_hip_ctx *ctx, const void *W_gate, const void *W_up, const void *panel,
+                                                            void *panel_out, int32_t K, int32_t N, int32_t M) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, W_gate && W_up && panel && panel_out, GALOIS_HIP_E_NULL, "mul_mat_q4_0_swiglu_f16_panel");
+    GH_REQUIRE(ctx, gemm_panel_shape_ok(K, M) && gemm_panel_shape_ok(N, M), GALOIS_HIP_E_SHAPE,
+               "mul_mat_q4_0_swiglu_f16_panel: K and N positive multiples of 256, (M + 16) * K and (M + 16) * N below 2^31");
+    GH_REQUIRE(ctx, gh_aligned(W_gate, 16) && gh_aligned(W_up, 16) && gh_aligned(panel, 16) && gh_aligned(panel_out, 16), GALOIS_HIP_E_ALIGN,
+               "mul_mat_q4_0_swiglu_f16_panel: 16-byte aligned operands");
+    GH_REQUIRE(ctx, panel != panel_out, GALOIS_HIP_E_SHAPE, "mul_mat_q4_0_swiglu_f16_panel: the two panels are distinct");
+    GH_BIND(ctx);
+    gemm_mats mats = {};
+    mats.W[0] = (const uint8_t *)W_gate, mats.W[1] = (const uint8_t *)W_up, mats.N[0] = mats.N[1] = N;
+    for (int j = 0; j < GEMM_MAX_MATS; j++) mats.col0[j] = 0x7FFFFFFF;
+    mats.n_total = 96 * ((N + 47) / 48);
+    mats.swiglu_out = static_cast<_Float16 *>(panel_out);
+    const int32_t st = gemm_launch<96>(ctx, mats, (const _Float16 *)panel, K, M);
+    if (st != GALOIS_HIP_OK) return st;
+    GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_swiglu_f16_panel launch");
 }

@@ -81,7 +81,7 @@ class LlamaDecoder {
     Tensor ssq_, ssq1_;  // partial sums of squares of x and x1 (fused = 4)
     struct Prefill {  // intermediates of prefill(), for up to `rows` tokens attending over up to `keys` positions
         size_t rows = 0, keys = 0;
-        Tensor tok, pos, x, x1, q, k, v, qr, kr, q3, s, p, o, ao, g, u, panel_e, panel_f, split_ws;
+        Tensor tok, pos, x, x1, q, k, v, qr, kr, q3, s, p, o, ao, panel_e, panel_f, split_ws;
     };
     GResult prefill_buffers(size_t n, size_t keys);
     Prefill pf_;
@@ -133,6 +133,9 @@ GResult galois_matmul_panel_add(const Tensor &w, const Tensor &panel, const Tens
 GResult galois_attn_decode(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor &v, Tensor &k_cache,
                            Tensor &v_cache, const Tensor &pos, Tensor &out, size_t n_head, int32_t n_past, float scale);
 
+// panel_out = the panel of silu(w_gate . x) * (w_up . x) for x given as `panel` ([K, M] operand), one launch
+// (galois_hip_mul_mat_q4_0_swiglu_f16_panel); w_gate, w_up [K, N] Q4_0, panel_out of galois_panel_elems(N, M) elements.
+GResult galois_matmul_swiglu_panel(const Tensor &w_gate, const Tensor &w_up, const Tensor &panel, Tensor &panel_out, size_t K, size_t M);
 // The product alone as its one or two shares of k (galois_hip_mul_mat_q4_0_f16_panel_shares): shares is an F32 tensor of
 // at least N * M elements (2 * N * M let a narrow matrix run as two shares); *n_shares says how many partial results
 // it now holds, N * M elements apart.

@@ -109,6 +109,25 @@ GResult galois_matmul_panel_add(const Tensor &w, const Tensor &panel, const Tens
         workspace ? (int64_t)(workspace->dim().elem_count() * sizeof(float)) : 0));
 }
 
+GResult galois_matmul_swiglu_panel(const Tensor &w_gate, const Tensor &w_up, const Tensor &panel, Tensor &panel_out, size_t K, size_t M) {
+    if (!panel.device().is_gpu() || panel.dtype() != GGmlType::F16 || panel.dim().elem_count() < galois_panel_elems(K, M))
+        return err(GError::ShapeError, "galois_matmul_swiglu_panel: an F16 Gpu panel of galois_panel_elems(K, M) elements");
+    const auto &dev = panel.device().gpu;
+    for (const Tensor *t : {&w_gate, &w_up, (const Tensor *)&panel_out})
+        if (!t->device().is_gpu() || t->device().gpu != dev)
+            return err(GError::Unimplemented, "galois_matmul_swiglu_panel: Gpu tensors on the panel's device");
+    const size_t N = w_gate.dim().shape[1];
+    for (const Tensor *w : {&w_gate, &w_up})
+        if (w->dtype() != GGmlType::Q4_0 || !w->dim().ggml_is_contiguous(w->dtype()) || w->dim().shape[0] != K ||
+            w->dim().elem_count() != K * N)
+            return err(GError::ShapeError, "galois_matmul_swiglu_panel: w_gate and w_up contiguous Q4_0 [K, N]");
+    if (panel_out.dtype() != GGmlType::F16 || !panel_out.dim().ggml_is_contiguous(panel_out.dtype()) ||
+        panel_out.dim().elem_count() < galois_panel_elems(N, M) || panel_out.data() == panel.data())
+        return err(GError::ShapeError, "galois_matmul_swiglu_panel: panel_out a second F16 tensor of galois_panel_elems(N, M) elements");
+    return dev->check(galois_hip_mul_mat_q4_0_swiglu_f16_panel(dev->ctx(), w_gate.data(), w_up.data(), panel.data(), panel_out.data(),
+                                                               (int32_t)K, (int32_t)N, (int32_t)M));
+}
+
 GResult galois_matmul_panel_shares(const Tensor &w, const Tensor &panel, Tensor &shares, size_t K, size_t M, int32_t *n_shares) {
     if (!n_shares) return err(GError::Unexpected, "galois_matmul_panel_shares: n_shares is required");
     if (!panel.device().is_gpu() || panel.dtype() != GGmlType::F16 || panel.dim().elem_count() < galois_panel_elems(K, M))
@@ -205,8 +224,6 @@ GResult LlamaDecoder::prefill_buffers(size_t n, size_t keys) {
         G_TRY(mk(&b.s, F32, dev_, kk, rows, H));
         G_TRY(mk(&b.p, F32, dev_, kk, rows, H));
     }
-    G_TRY(mk(&b.g, F32, dev_, F, rows));
-    G_TRY(mk(&b.u, F32, dev_, F, rows));
     G_TRY(mk(&b.panel_e, GGmlType::F16, dev_, galois_panel_elems(E, rows)));
     G_TRY(mk(&b.panel_f, GGmlType::F16, dev_, galois_panel_elems(F, rows)));
     G_TRY(mk(&b.split_ws, F32, dev_, 2 * E * rows));
@@ -229,9 +246,9 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
     Prefill &b = pf_;
     galois_hip_ctx *ctx = dev_.gpu->ctx();
     // views of the buffers at this call's n and L (the buffers may be larger)
-    Tensor tok, pos, x, x1, q, k, v, ao, qr, kr, q3, o, s, p, g, u;
+    Tensor tok, pos, x, x1, q, k, v, ao, qr, kr, q3, o, s, p;
     {
-        const size_t one[1] = {n}, en[2] = {E, n}, fn[2] = {F, n}, dhn[3] = {D, H, n}, dnh[3] = {D, n, H}, lnh[3] = {L, n, H};
+        const size_t one[1] = {n}, en[2] = {E, n}, dhn[3] = {D, H, n}, dnh[3] = {D, n, H}, lnh[3] = {L, n, H};
         G_TRY(b.tok.view(0, 1, one, &tok));
         G_TRY(b.pos.view(0, 1, one, &pos));
         for (auto pr : {std::make_pair(&b.x, &x), std::make_pair(&b.x1, &x1), std::make_pair(&b.q, &q),
@@ -246,8 +263,6 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
             G_TRY(b.s.view(0, 3, lnh, &s));
             G_TRY(b.p.view(0, 3, lnh, &p));
         }
-        G_TRY(b.g.view(0, 2, fn, &g));
-        G_TRY(b.u.view(0, 2, fn, &u));
     }
     std::vector<int32_t> positions(n);
     for (size_t i = 0; i < n; i++) positions[i] = n_past + (int32_t)i;
@@ -331,10 +346,9 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
         int32_t shares = 0;
         G_TRY(galois_matmul_panel_shares(l.wo, b.panel_e, b.split_ws, E, n, &shares));
         G_TRY(galois_add_rms_norm_mul_panel(b.split_ws, shares, &x, x1, l.ffn_norm, b.panel_e, hp_.rms_eps)); ops += 2;
-        // feed-forward block: gate | up in one launch, SwiGLU -> panel, down as shares; the adding pass writes the next
+        // feed-forward block: gate | up with the SwiGLU in one launch -> panel, down as shares; the adding pass writes the next
         // layer's attention norm (after the last layer there is no next norm: the plain adding pass)
-        G_TRY(galois_matmul_panel({{&l.w_gate, &g}, {&l.w_up, &u}}, b.panel_e, E, n));
-        G_TRY(galois_silu_mul_panel(g, u, b.panel_f)); ops += 2;
+        G_TRY(galois_matmul_swiglu_panel(l.w_gate, l.w_up, b.panel_e, b.panel_f, E, n)); ops++;
         if (li + 1 < layers_.size()) {
             G_TRY(galois_matmul_panel_shares(l.w_down, b.panel_f, b.split_ws, F, n, &shares));
             G_TRY(galois_add_rms_norm_mul_panel(b.split_ws, shares, &x1, x, layers_[li + 1].attn_norm, b.panel_e, hp_.rms_eps)); ops += 2;

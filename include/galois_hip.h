@@ -372,6 +372,16 @@ int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, const void *W
                                               float *Y, int32_t K, int32_t N, int32_t M, void *workspace,
                                               int64_t workspace_bytes);
 
+/* The gate and up projections of a feed-forward block and the SwiGLU between them and the down projection in one
+ * launch: panel_out = the fp16 panel of silu(W_gate . x) * (W_up . x) ([N, M] operand, galois_hip_f16_panel_bytes(N, M)
+ * bytes) for x given as `panel` ([K, M] operand) -- galois_hip_mul_mat_q4_0_f16_panel on the two matrices followed by
+ * galois_hip_silu_mul_f16_panel (CudaMatMul x 2, silu_f32, mul_f32) without the two f32 results ever reaching memory:
+ * a tile of the launch holds 48 columns of each matrix, so both products of an element meet in one wave's registers.
+ * The products are the same bits as the two-call form's and the SwiGLU is the same expression; its compiled form may
+ * fuse 1 + exp(-g) differently, so single elements can differ by one unit in the last place of fp16.  W_gate, W_up: [N rows][K / 32] Q4_0 blocks; K and N multiples of 256. */
+int32_t galois_hip_mul_mat_q4_0_swiglu_f16_panel(galois_hip_ctx *ctx, const void *W_gate, const void *W_up, const void *panel,
+                                                 void *panel_out, int32_t K, int32_t N, int32_t M);
+
 /* The product of galois_hip_mul_mat_q4_0_f16_panel_add alone, as the shares of k it is computed in, for a caller whose
  * next op does the adding (galois_hip_add_rms_norm_mul_f16_panel below): *n_shares = 1 or 2 partial results [M][N] f32
  * at shares and shares + M * N, whose sum (in that order) is W . panel.  Two only when that pays for the shape

@@ -161,6 +161,39 @@ def test_shares_then_adding_pass_fused_with_the_next_norm(dev, m, k, n, with_res
         dev.free(b)
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 4096, 11008), (130, 256, 512), (33, 768, 256), (300, 1024, 2816), (1, 512, 768)])
+def test_gate_up_and_swiglu_in_one_launch(dev, m, k, n):
+    """The panel of silu(Wg . x) * (Wu . x) from one launch against the panel that the two-matrix matmul followed by
+    the SwiGLU-to-panel call writes: the products are the same bits and the SwiGLU the same expression, but the compiler
+    is free to fuse 1 + exp(-g) into the exponential's last step in one kernel and not in the other, so a few elements
+    (here: fewer than one in a thousand) differ by one unit in the last place of fp16; rows past m are zeros; the down
+    projection on the panel meets twice the prefill bar against the oracle's ops on the oracle's activations."""
+    x, (wg, wu) = _case(m + k + n + 7, m, k, [n, n])
+    rng = np.random.default_rng(k + n)
+    n_out = 160
+    wd = oracle.quantize_q4_0((rng.standard_normal((n_out, n)) * 0.02).astype(np.float32))
+    xb, gb, ub, db = dev.upload(x), dev.upload(wg), dev.upload(wu), dev.upload(wd)
+    pb, _ = _panel(dev, k, m)
+    dev.f32_to_f16_panel(xb, pb, k, m)
+    p_ref, nb = _panel(dev, n, m)
+    p_got, _ = _panel(dev, n, m)
+    dev.upload(np.full(nb // 4, 7.5, np.float32), p_got)
+    yg, yu, yd = dev.alloc(m * n * 4), dev.alloc(m * n * 4), dev.alloc(m * n_out * 4)
+    dev.mul_mat_q4_0_f16_panel([(gb, yg, n), (ub, yu, n)], pb, k, m)
+    dev.silu_mul_f16_panel(yg, yu, p_ref, n, m)
+    dev.mul_mat_q4_0_swiglu_f16_panel(gb, ub, pb, p_got, k, n, m)
+    got, ref = _untile(dev.download(p_got, np.uint8, nb), m, n), _untile(dev.download(p_ref, np.uint8, nb), m, n)
+    assert _ulps_f16(got[:m], ref[:m]) <= 1.0
+    assert np.count_nonzero(got[:m] != ref[:m]) <= max(1, got[:m].size // 1000)
+    assert np.all(got[m:] == 0)
+    dev.mul_mat_q4_0_f16_panel([(db, yd, n_out)], p_got, n, m)
+    act = oracle.mul(oracle.silu(oracle.mul_mat_q4_0_f32(wg, x)).reshape(-1), oracle.mul_mat_q4_0_f32(wu, x).reshape(-1)).reshape(m, n)
+    emax, el2 = npref.rel_err(dev.download(yd, np.float32, (m, n_out)), oracle.mul_mat_q4_0_f32(wd, act))
+    assert emax < 2 * TOL and el2 < 2 * TOL, (emax, el2)      # two products and a rounding to fp16 in a row
+    for b in (xb, gb, ub, db, pb, p_ref, p_got, yg, yu, yd):
+        dev.free(b)
+
+
 def _ulps_f16(a, b):
     """Largest distance between two float16 arrays in units of the last place of the larger magnitude."""
     a32, b32 = a.astype(np.float32), b.astype(np.float32)
