@@ -570,6 +570,13 @@ def main():
         tpanel("matmul_512x4096x11008", lambda: dev.mul_mat_q4_0_f16_panel([(wp, yp, n)], pb, k, m), 2.0 * m * k * n)
         tpanel("gate_up_one_launch_512x4096x2x11008",
                lambda: dev.mul_mat_q4_0_f16_panel([(w, y, n) for w, y in zip(w2, y2)], pb, k, m), 2 * 2.0 * m * k * n)
+        pf2 = dev.alloc(dev.f16_panel_bytes(n, m))
+        tpanel("gate_up_one_launch_then_swiglu_to_panel",
+               lambda: (dev.mul_mat_q4_0_f16_panel([(w, y, n) for w, y in zip(w2, y2)], pb, k, m),
+                        dev.silu_mul_f16_panel(y2[0], y2[1], pf2, n, m)), 2 * 2.0 * m * k * n)
+        tpanel("gate_up_and_swiglu_one_launch_512x4096x2x11008",
+               lambda: dev.mul_mat_q4_0_swiglu_f16_panel(w2[0], w2[1], pb, pf2, k, n, m), 2 * 2.0 * m * k * n)
+        dev.free(pf2)
         tpanel("qkv_one_launch_512x4096x3x4096",
                lambda: dev.mul_mat_q4_0_f16_panel([(w, y, 4096) for w, y in zip(w3, y3)], pb, k, m), 3 * 2.0 * m * k * 4096)
         tpanel("qkv_three_f32_calls_512x4096x4096",

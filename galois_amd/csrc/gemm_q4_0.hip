@@ -633,6 +633,9 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
         // (silu_f32 then mul_f32, unary.cu:1-10, mul.cu:3-12, with the arithmetic of f32_to_f16_tiles<true>) goes
         // to the panel as fp16: element (m, n) lies in tile (m / 16, n / 32) of 1 KB, 16-byte piece ((n % 32) / 8) * 16
         // + m % 16, at n % 8.  Rows of the panel past M were zeros in the input panel, so their products are zeros.
+        // The exponential and the reciprocal are the hardware's (v_exp_f32, v_rcp_f32: about one unit in the last place
+        // of f32 each, far below the fp16 rounding that follows); four neighbouring lanes hold four neighbouring
+        // columns of a row, which lane % 4 == 0 gathers over the quad and stores as one 8-byte piece.
         const int N = mats.N[0], m_pad = (M + 15) & ~15;
         unsigned char *out = reinterpret_cast<unsigned char *>(mats.swiglu_out);
 #pragma unroll
@@ -645,9 +648,14 @@ __device__ __forceinline__ void gemm_consumer(const _Float16 *smem, const _Float
                 for (int e = 0; e < 4; e++) {
                     const int m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + e;
                     const float g = acc[i][j][e], u = acc[i][j + 3 < NF ? j + 3 : j][e];
-                    const _Float16 h = (_Float16)(g / (1.0f + expf(-g)) * u);
-                    if (m < m_pad && n < N)
-                        *reinterpret_cast<_Float16 *>(out + (size_t)(m >> 4) * (size_t)(N >> 5) * 1024 + col_at + (size_t)(m & 15) * 16) = h;
+                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504088896340736f));
+                    const uint32_t h = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)((g * sig) * u));
+                    // quad_perm [1,0,3,2] then [2,3,0,1]: lane 4q ends up with the four halfs of its quad in column order
+                    const uint32_t pair = h | ((uint32_t)__builtin_amdgcn_update_dpp(0, (int)h, 0xB1, 0xF, 0xF, false) << 16);
+                    const uint32_t pair2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pair, 0x4E, 0xF, 0xF, false);
+                    if ((lane & 3) == 0 && m < m_pad && n < N)
+                        *reinterpret_cast<uint2 *>(out + (size_t)(m >> 4) * (size_t)(N >> 5) * 1024 + col_at + (size_t)(m & 15) * 16) =
+                            make_uint2(pair, pair2);
                 }
         }
         return;
