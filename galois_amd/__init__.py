@@ -303,6 +303,11 @@ class Device:
         self._check(self._lib.galois_hip_add_rms_norm_mul_f16_panel(self._ctx, _ptr(a), _ptr(b), _ptr(c), _ptr(sum_out), _ptr(weight),
                                                                     _ptr(panel), ncols, nrows, eps))
 
+    def rope_qk_append(self, q, k, v, q_out, k_rows, v_rows, kv_f16, head_dim, n_head, n_tokens, pos, freq_scale, theta_scale):
+        """rope of q (to q_out) and of k (to the cache rows k_rows) and, when v is given, v to v_rows, one launch."""
+        self._check(self._lib.galois_hip_rope_qk_append(self._ctx, _ptr(q), _ptr(k), _ptr(v), _ptr(q_out), _ptr(k_rows), _ptr(v_rows),
+                                                        int(kv_f16), head_dim, n_head, n_tokens, _ptr(pos), freq_scale, theta_scale))
+
     def attn_prefill(self, q, k_cache, v_cache, out, out_panel, n_head, head_dim, n_tokens, n_past, scale, kv_f16=False):
         """Causal attention of n_tokens rows of q over caches that already hold positions 0 .. n_past + n_tokens - 1;
         the result goes to out (f32) or out_panel (fp16 panel), the other is None."""

@@ -82,6 +82,7 @@ PROTOTYPES = {
     "galois_hip_mul_mat_q4_0_swiglu_f16_panel": (i32, [c_ctx, vp, vp, vp, vp, i32, i32, i32]),
     "galois_hip_mul_mat_q4_0_f16_panel_shares": (i32, [c_ctx, vp, vp, vp, C.c_int64, i32, i32, i32, C.POINTER(i32)]),
     "galois_hip_add_rms_norm_mul_f16_panel": (i32, [c_ctx, vp, vp, vp, vp, vp, vp, i32, i32, f32]),
+    "galois_hip_rope_qk_append": (i32, [c_ctx, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, f32]),
     "galois_hip_attn_prefill_f32": (i32, [c_ctx, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]),
     "galois_hip_attn_prefill_f16kv": (i32, [c_ctx, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]),
     "galois_hip_qkv_attn_decode_f16kv": (i32, [c_ctx, C.POINTER(GemvItem), vp, vp, vp, i32, i32, i32, vp, f32, f32, f32, i32]),

@@ -188,6 +188,54 @@ __global__ __launch_bounds__(kRopeThreads) void rope_rows4(const float *__restri
     for (; r < row_hi; r += RS) st4(y + (size_t)r * ncols + 4 * c4, rot(ld4(x + (size_t)r * ncols + 4 * c4)));
 }
 
+
+// rope_custom of the q and the k rows of many tokens and the append of k and v to the cache rows of those tokens, one
+// launch: one workgroup per token; sin / cos of a lane's two pairs are computed once (the formula of rope_rows4) and
+// serve the token's q rows and k rows alike.  q goes rotated to qo (f32); k rotated to kd and, when v is given, v
+// unchanged to vd: f32, or f16 rounded to nearest even (cpy_f32_f16, cpy.cu:79-156, into an f16 cache).
+template <int LPR, bool KV16>
+__global__ __launch_bounds__(kRopeThreads) void rope_qk_append_rows4(const float *__restrict__ q, const float *__restrict__ k,
+                                                                     const float *__restrict__ v, float *__restrict__ qo,
+                                                                     void *__restrict__ kd, void *__restrict__ vd, int head_dim,
+                                                                     int n_head, const int32_t *__restrict__ pos,
+                                                                     float freq_scale, float theta_scale) {
+    constexpr int RPW = 64 / LPR;                  // rows per wave-load
+    constexpr int RS = (kRopeThreads / 64) * RPW;  // rows per workgroup-load
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / LPR, c4 = lane % LPR;
+    if (c4 * 4 >= head_dim) return;
+    const size_t tok = (size_t)blockIdx.x * n_head * head_dim;
+    const float p0 = (float)pos[blockIdx.x] * freq_scale;
+    float s0, c0, s1, c1;
+    sincosf(p0 * powf(theta_scale, (float)(2 * c4)), &s0, &c0);
+    sincosf(p0 * powf(theta_scale, (float)(2 * c4 + 1)), &s1, &c1);
+    auto rot = [&](float4 x) {
+        return make_float4(__builtin_fmaf(x.x, c0, -(x.y * s0)), __builtin_fmaf(x.x, s0, x.y * c0),
+                           __builtin_fmaf(x.z, c1, -(x.w * s1)), __builtin_fmaf(x.z, s1, x.w * c1));
+    };
+    auto put = [&](void *dst, size_t at, float4 x) {
+        if (KV16) {
+            // the rotation's f32 results first, then their rounding to f16, as the two ops would do it: left to the
+            // compiler the multiply-add and the conversion become one instruction with a single rounding
+            asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
+            typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store(h4{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w},
+                                        reinterpret_cast<h4 *>(static_cast<_Float16 *>(dst) + at));
+        } else {
+            st4(static_cast<float *>(dst) + at, x);
+        }
+    };
+    for (int r = wave * RPW + sub; r < n_head; r += RS) {
+        const size_t at = tok + (size_t)r * head_dim + 4 * c4;
+        const float4 a = ld4(q + at), b = ld4(k + at);
+        float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v) c = ld4(v + at);
+        st4(qo + at, rot(a));
+        put(kd, at, rot(b));
+        if (v) put(vd, at, c);
+    }
+}
+
 __global__ __launch_bounds__(kRopeThreads) void rope_rows(const float *__restrict__ x, float *__restrict__ y,
                                                           int ncols, int nrows, const int32_t *__restrict__ pos,
                                                           float freq_scale, int p_delta_rows, float theta_scale) {
@@ -380,6 +428,33 @@ int32_t galois_hip_rope_f32(galois_hip_ctx *ctx, const float *x, float *dst, int
     hipLaunchKernelGGL(rope_rows, dim3(groups), dim3(kRopeThreads), 0, ctx->stream, x, dst, ncols, nrows, pos,
                        freq_scale, p_delta_rows, theta_scale);
     GH_LAUNCH_CHECK(ctx, "rope_f32 launch");
+}
+
+int32_t galois_hip_rope_qk_append(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, float *q_out, void *k_rows,
+                                  void *v_rows, int32_t kv_f16, int32_t head_dim, int32_t n_head, int32_t n_tokens,
+                                  const int32_t *pos, float freq_scale, float theta_scale) {
+    GH_REQUIRE_CTX(ctx);
+    GH_REQUIRE(ctx, q && k && q_out && k_rows && pos && ((v != nullptr) == (v_rows != nullptr)), GALOIS_HIP_E_NULL,
+               "rope_qk_append: q, k, q_out, k_rows, pos; v and v_rows together or neither");
+    GH_REQUIRE(ctx, head_dim > 0 && head_dim % 4 == 0 && head_dim <= 256 && n_head > 0 && n_tokens > 0, GALOIS_HIP_E_SHAPE,
+               "rope_qk_append: head_dim a multiple of 4 up to 256, n_head and n_tokens positive");
+    GH_REQUIRE(ctx, gh_aligned(q, 16) && gh_aligned(k, 16) && gh_aligned(v, 16) && gh_aligned(q_out, 16) && gh_aligned(k_rows, 16) &&
+                        gh_aligned(v_rows, 16) && gh_aligned(pos, 4), GALOIS_HIP_E_ALIGN, "rope_qk_append: 16-byte aligned tensors");
+    GH_BIND(ctx);
+#define GH_ROPE_QK(LPR)                                                                                                      \
+    do {                                                                                                                     \
+        if (kv_f16)                                                                                                          \
+            hipLaunchKernelGGL((rope_qk_append_rows4<LPR, true>), dim3(n_tokens), dim3(kRopeThreads), 0, ctx->stream, q, k, v, q_out, \
+                               k_rows, v_rows, head_dim, n_head, pos, freq_scale, theta_scale);                              \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((rope_qk_append_rows4<LPR, false>), dim3(n_tokens), dim3(kRopeThreads), 0, ctx->stream, q, k, v, q_out, \
+                               k_rows, v_rows, head_dim, n_head, pos, freq_scale, theta_scale);                              \
+    } while (0)
+    if (head_dim <= 64) GH_ROPE_QK(16);
+    else if (head_dim <= 128) GH_ROPE_QK(32);
+    else GH_ROPE_QK(64);
+#undef GH_ROPE_QK
+    GH_LAUNCH_CHECK(ctx, "rope_qk_append launch");
 }
 
 int32_t galois_hip_soft_max_f32(galois_hip_ctx *ctx, const float *x, float *dst, int32_t ncols, int32_t nrows) {

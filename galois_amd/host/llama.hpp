@@ -145,6 +145,12 @@ GResult galois_matmul_panel_shares(const Tensor &w, const Tensor &panel, Tensor 
 GResult galois_add_rms_norm_mul_panel(const Tensor &shares, int32_t n_shares, const Tensor *residual, Tensor &sum_out,
                                       const Tensor &weight, Tensor &panel, float eps);
 
+// rope_custom (mode 0, n_dims = head_dim) of q and k ([head_dim, n_head, n] f32, positions pos) and the append to the
+// caches' rows of those tokens, one launch (galois_hip_rope_qk_append): q rotated to q_out; k rotated to k_rows and, when
+// v is given, v to v_rows -- contiguous views of the caches' rows, [n_embd, n], both F32 or both F16.
+GResult galois_rope_qk_append(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor *v, const Tensor &pos,
+                              Tensor &q_out, Tensor &k_rows, Tensor *v_rows);
+
 // Causal attention of all rows of q ([n_embd, n] f32, rotated) over caches ([n_embd, n_ctx], both f32 or both f16) that
 // already hold positions 0 .. n_past + n - 1, in one launch (galois_hip_attn_prefill_f32 / _f16kv; heads of 128).
 // dst is either an F32 tensor [n_embd, n] or an F16 panel of galois_panel_elems(n_embd, n) elements.

@@ -166,6 +166,32 @@ GResult galois_add_rms_norm_mul_panel(const Tensor &shares, int32_t n_shares, co
                                                             (const float *)weight.data(), panel.data(), (int32_t)K, (int32_t)M, eps));
 }
 
+GResult galois_rope_qk_append(const RopeCustomOption &op, const Tensor &q, const Tensor &k, const Tensor *v, const Tensor &pos,
+                              Tensor &q_out, Tensor &k_rows, Tensor *v_rows) {
+    if ((v == nullptr) != (v_rows == nullptr)) return err(GError::Unexpected, "galois_rope_qk_append: v and v_rows together or neither");
+    const auto &dev = q.device().gpu;
+    for (const Tensor *t : {&q, &k, v, &pos, (const Tensor *)&q_out, (const Tensor *)&k_rows, (const Tensor *)v_rows})
+        if (t && (!t->device().is_gpu() || t->device().gpu != dev || !t->dim().ggml_is_contiguous(t->dtype())))
+            return err(GError::Unimplemented, "galois_rope_qk_append: contiguous Gpu tensors on one device");
+    if (op.mode != 0) return err(GError::Unimplemented, "galois_rope_qk_append: mode 0");
+    if (q.dtype() != GGmlType::F32 || k.dtype() != GGmlType::F32 || q_out.dtype() != GGmlType::F32 || (v && v->dtype() != GGmlType::F32) ||
+        pos.dtype() != GGmlType::I32)
+        return err(GError::Unimplemented, "galois_rope_qk_append: F32 q, k, v, q_out and I32 positions");
+    const GGmlType ct = k_rows.dtype();
+    if ((ct != GGmlType::F32 && ct != GGmlType::F16) || (v_rows && v_rows->dtype() != ct))
+        return err(GError::Unimplemented, "galois_rope_qk_append: cache rows both F32 or both F16");
+    const size_t D = q.dim().shape[0], H = q.dim().shape[1], n = q.dim().shape[2], total = D * H * n;
+    if (q.dim().n_dims != 3 || op.n_dims != D || D % 4 != 0 || D > 256 || pos.dim().shape[0] != n)
+        return err(GError::ShapeError, "galois_rope_qk_append: q [head_dim, n_head, n] with n_dims = head_dim (a multiple of 4 up to 256), one position per token");
+    for (const Tensor *t : {&k, v, (const Tensor *)&q_out, (const Tensor *)&k_rows, (const Tensor *)v_rows})
+        if (t && t->dim().elem_count() != total) return err(GError::ShapeError, "galois_rope_qk_append: every tensor has q's element count");
+    const float theta_scale = powf(op.freq_base, -2.0f / (float)op.n_dims);  // as galois_rope_custom derives it (src/cuda.rs:1327)
+    return dev->check(galois_hip_rope_qk_append(dev->ctx(), (const float *)q.data(), (const float *)k.data(),
+                                                v ? (const float *)v->data() : nullptr, (float *)q_out.data(), k_rows.data(),
+                                                v_rows ? v_rows->data() : nullptr, ct == GGmlType::F16, (int32_t)D, (int32_t)H, (int32_t)n,
+                                                (const int32_t *)pos.data(), op.freq_scale, theta_scale));
+}
+
 GResult galois_attn_prefill(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &dst, size_t n_head,
                             int32_t n_past, float scale) {
     for (const Tensor *t : {&q, &k_cache, &v_cache, (const Tensor *)&dst})
@@ -291,8 +317,17 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
         Tensor k_rows, v_rows;  // rows n_past .. n_past + n - 1 of both caches: one contiguous piece each
         G_TRY(l.k_cache.view(P * E, 2, en, &k_rows));
         G_TRY(l.v_cache.view(P * E, 2, en, &v_rows));
-        if (!hp_.kv_f16) {
-            // f32 caches take the values straight from the product and the keys straight from the rotation
+        if (D % 4 == 0 && D <= 256) {
+            // both rotations and the append in one launch; an f32 cache takes the values straight from the product
+            if (!hp_.kv_f16) {
+                G_TRY(galois_matmul_panel({{&l.wq, &q}, {&l.wk, &k}, {&l.wv, &v_rows}}, b.panel_e, E, n));
+                G_TRY(galois_rope_qk_append(rope, q_heads, k_heads, nullptr, pos, qr, k_rows, nullptr));
+            } else {
+                G_TRY(galois_matmul_panel({{&l.wq, &q}, {&l.wk, &k}, {&l.wv, &v}}, b.panel_e, E, n));
+                G_TRY(galois_rope_qk_append(rope, q_heads, k_heads, &v, pos, qr, k_rows, &v_rows));
+            }
+            ops += 2;
+        } else if (!hp_.kv_f16) {
             Tensor kr_cache;
             const size_t dhn[3] = {D, H, n};
             G_TRY(k_rows.view(0, 3, dhn, &kr_cache));

@@ -397,6 +397,19 @@ int32_t galois_hip_mul_mat_q4_0_f16_panel_shares(galois_hip_ctx *ctx, const void
 int32_t galois_hip_add_rms_norm_mul_f16_panel(galois_hip_ctx *ctx, const float *a, const float *b, const float *c, float *sum_out,
                                               const float *weight, void *panel, int32_t ncols, int32_t nrows, float eps);
 
+/* What a prefill does between its q | k | v products and its attention, one launch instead of two to four:
+ * rope_custom (mode 0, n_dims = head_dim) of q and of k for n_tokens tokens -- rope_f32 twice, src/cuda.rs:1257-1356,
+ * with the same arithmetic, q_out and the rotated k bit-equal to galois_hip_rope_f32's -- and the append of the rotated
+ * k and (when v is given) of v to the cache rows of those tokens (cpy_f32_f32 / cpy_f32_f16, src/cuda.rs:1382-1595):
+ *   q, k, v: [n_tokens][n_head * head_dim] f32; pos: the tokens' positions (int32, on the device);
+ *   q_out: [n_tokens][n_head * head_dim] f32; k_rows, v_rows: the caches' rows of these tokens, contiguous
+ *   [n_tokens][n_head * head_dim], f32 (kv_f16 = 0) or f16 rounded to nearest even (kv_f16 = 1).
+ * v and v_rows are both null when the values are already in place (an f32 cache can take them from the product).
+ * head_dim a multiple of 4 up to 256; 16-byte aligned tensors. */
+int32_t galois_hip_rope_qk_append(galois_hip_ctx *ctx, const float *q, const float *k, const float *v, float *q_out, void *k_rows,
+                                  void *v_rows, int32_t kv_f16, int32_t head_dim, int32_t n_head, int32_t n_tokens,
+                                  const int32_t *pos, float freq_scale, float theta_scale);
+
 /* Causal attention of n_tokens query rows over a KV cache in ONE launch: what a prefill issues per layer as
  * cpy(q -> [D, M, H]), matmul(K^T, q), scale, soft_max under the causal mask, matmul(V, p), cpy(-> [D, H, M])
  * (CudaMatMul src/cuda.rs:867-992, scale and soft_max src/cuda.rs:1597-1663 and 1257-1356, cpy src/cuda.rs:1382-1595),

@@ -96,6 +96,35 @@ def test_rope_vs_oracle(dev, t, h, hd, p0):
     assert np.array_equal(got0, x)
 
 
+@pytest.mark.parametrize("kv_f16", [False, True])
+@pytest.mark.parametrize("with_v", [False, True])
+@pytest.mark.parametrize("t,h,hd,p0", [(1, 1, 4, 0), (3, 5, 64, 100), (77, 32, 128, 1971), (512, 32, 128, 0), (4, 7, 256, 17), (9, 3, 36, 5)])
+def test_rope_of_q_and_k_with_the_append_in_one_launch(dev, t, h, hd, p0, with_v, kv_f16):
+    """galois_hip_rope_qk_append against the calls it replaces: q_out and the rotated k are galois_hip_rope_f32's bits
+    (rope_f32 itself is held to the oracle above); into an f16 cache k and v arrive as numpy's round-to-nearest-even of
+    those f32 values; nothing is written past the rows of the call."""
+    rng = np.random.default_rng(t + h + hd + p0)
+    e = h * hd
+    q, k, v = (rng.standard_normal((t * h, hd)).astype(np.float32) for _ in range(3))
+    pos = np.arange(p0, p0 + t, dtype=np.int32)
+    ts = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    want_q, want_k = _rope(dev, q, pos, 1.0, h, ts), _rope(dev, k, pos, 1.0, h, ts)
+    ct = np.float16 if kv_f16 else np.float32
+    qb, kb, vb, pb = dev.upload(q), dev.upload(k), dev.upload(v), dev.upload(pos)
+    qo = dev.upload(np.full(t * e + 8, 7.5, np.float32))
+    kd, vd = dev.upload(np.full(t * e + 8, 7.5, ct)), dev.upload(np.full(t * e + 8, 7.5, ct))
+    dev.rope_qk_append(qb, kb, vb if with_v else None, qo, kd, vd if with_v else None, kv_f16, hd, h, t, pb, 1.0, ts)
+    got_q = dev.download(qo, np.float32, t * e + 8)
+    got_k, got_v = dev.download(kd, ct, t * e + 8), dev.download(vd, ct, t * e + 8)
+    assert np.array_equal(got_q[:t * e].view(np.uint32), want_q.reshape(-1).view(np.uint32))
+    assert np.array_equal(got_k[:t * e], want_k.reshape(-1).astype(ct))
+    assert np.array_equal(got_v[:t * e], v.reshape(-1).astype(ct) if with_v else np.full(t * e, 7.5, ct))
+    for tail in (got_q[t * e:], got_k[t * e:], got_v[t * e:]):
+        assert np.all(tail == 7.5)
+    for b in (qb, kb, vb, pb, qo, kd, vd):
+        dev.free(b)
+
+
 # ------------------------------------------------------------------ softmax
 def _soft(dev, x, causal=None):
     nrows, ncols = x.shape
