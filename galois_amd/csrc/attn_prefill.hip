@@ -5,12 +5,16 @@
 // soft_max src/cuda.rs:1257-1356, cpy src/cuda.rs:1382-1595) for heads of 128.  Scores never reach memory.
 //
 // Shape of the work on gfx950:
-//   - One workgroup of 4 waves per (head, 64 * QT consecutive queries); a wave owns 16 * QT queries for the whole walk
-//     over the keys and keeps their running maximum, running sum and the 16 x 128 output tile(s) in registers
-//     (the one-pass softmax: when the maximum grows, sum and output are rescaled by exp2(old - new)).
-//   - Keys are walked in blocks of 32.  The workgroup stages a block's K rows and V rows through LDS as fp16 (an f32
-//     cache is rounded here, the reference's convert_fp32_to_fp16 in front of its gemm_ex), double-buffered: the global
-//     loads of block b + 1 are in flight while block b is multiplied, one barrier per block.
+//   - One workgroup of 8 waves per (head, 64 * QT consecutive queries).  A wave owns 16 * QT queries and keeps their
+//     running maximum, running sum and the 16 x 128 output tile(s) in registers (the one-pass softmax: when the
+//     maximum grows, sum and output are rescaled by exp2(old - new)).  Two waves own the same queries: keys are walked
+//     in stages of 64, one wave multiplies the first 32-key block of every stage, the other the second, and at the end
+//     the second hands its maximum, sum and output to the first through LDS -- half the chain of dependent blocks per
+//     wave, and two waves per SIMD.
+//   - The workgroup stages K rows and V rows through LDS as fp16 (an f32 cache is rounded on the way, the reference's
+//     convert_fp32_to_fp16 in front of its gemm_ex), double-buffered: the global loads of stage s + 1 are in flight
+//     while stage s is multiplied (they are unconditional -- keys past the end point at the last live row and are
+//     zeroed on the way to LDS -- and stay raw in registers until then), one barrier per stage.
 //   - Both products use v_mfma_f32_16x16x32_f16 with the QUERY on the column side:
 //       S^T (16 keys x 16 queries) = K (A operand, rows = keys)  x  Q^T (B operand, 4 chunks of 32 dims),
 //       O^T (16 dims x 16 queries) = V^T (A operand, rows = dims) x  P^T (B operand, 32 keys),
@@ -351,9 +355,14 @@ int32_t pa_entry(galois_hip_ctx *ctx, const float *q, const void *k_cache, const
     a.q = q, a.kc = k_cache, a.vc = v_cache, a.out = out, a.panel = static_cast<_Float16 *>(out_panel);
     a.n = n_tokens, a.n_past = n_past, a.n_head = n_head;
     a.qscale = scale * 1.44269504088896340736f;
-    // 64 queries per workgroup while that does not leave more than four rounds of workgroups per CU; 128 beyond
-    const int64_t wg64 = ((int64_t)n_tokens + 63) / 64 * n_head;
-    const int qt = wg64 > (int64_t)ctx->n_cu * 4 ? 2 : 1;
+    // 64 queries per workgroup, or 128 (a wave then multiplies every K and V fragment it reads from LDS with two query
+    // tiles): the larger shape wins once the launch is bound by that traffic rather than by its dependent chains --
+    // four workgroups of 64 per CU or more, or two when every walk is long (as many cached positions as new rows, so
+    // that the causal walks differ by at most a factor of two).  Measured on 256 CUs, 32 heads, f32 cache, us for 64 /
+    // 128 queries: 512 rows 15.7 / 22.4, 1024 rows 31.0 / 37.4, 2048 rows 112 / 82.6, 1024 rows behind 1024 positions
+    // 83.7 / 72.0, 512 behind 1536 59.0 / 71.4; 8 heads x 4096 rows 100 / 124.
+    const int64_t wg64 = ((int64_t)n_tokens + 63) / 64 * n_head, cus = ctx->n_cu > 0 ? ctx->n_cu : 256;
+    const int qt = (wg64 >= 4 * cus || (wg64 >= 2 * cus && n_past >= n_tokens)) ? 2 : 1;
     a.tiles = (n_tokens + 64 * qt - 1) / (64 * qt);
     GH_REQUIRE(ctx, (int64_t)a.tiles * n_head < ((int64_t)1 << 31), GALOIS_HIP_E_SHAPE, "attn_prefill: too many workgroups");
     const hipError_t e = qt == 2 ? pa_launch<2>(ctx, a, kv16, out_panel != nullptr) : pa_launch<1>(ctx, a, kv16, out_panel != nullptr);

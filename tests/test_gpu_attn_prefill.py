@@ -7,7 +7,8 @@ The kernel's products take fp16 operands (q * scale * log2 e, keys, values, prob
 5e-3 where the scores reach +-100: rounding q and k to fp16 moves a score by about 2^-11 of its terms' size, and the
 exponential turns that absolute error into a relative one of the probabilities; the panel output is additionally the f32 output of the
 same call rounded to fp16.  Rows are independent of how the launch is cut into workgroups: the two workgroup shapes
-(64 or 128 queries) are compared with each other through a row count that selects the larger one.
+(64 or 128 queries) are compared with each other through a row count that selects the larger one, and the larger
+one is also the shape of the case of 1024 rows behind 1024 cached positions.
 """
 import numpy as np
 import pytest
@@ -56,7 +57,7 @@ def _inputs(seed, n_head, n, n_past, n_ctx, kv_f16, spread=1.0):
 
 @pytest.mark.parametrize("kv_f16", [False, True])
 @pytest.mark.parametrize("n_head,n,n_past", [(2, 1, 0), (2, 20, 0), (3, 77, 19), (32, 512, 0), (4, 64, 1), (2, 65, 31),
-                                             (1, 130, 700), (8, 300, 1000)])
+                                             (1, 130, 700), (8, 300, 1000), (32, 1024, 1024)])
 def test_attention_of_many_rows_against_the_op_sequence_in_f64(dev, n_head, n, n_past, kv_f16):
     e = n_head * D
     n_ctx = n_past + n + 5
