@@ -231,18 +231,21 @@ static GResult mk(Tensor *t, GGmlType ty, const Device &dev, size_t ne0, size_t 
 
 GResult LlamaDecoder::prefill_buffers(size_t n, size_t keys) {
     const size_t E = hp_.n_embd, F = hp_.n_ff, H = hp_.n_head, D = E / H;
-    const bool op_sequence = D != 128;  // the attention as single ops needs the scores and the permuted copies
+    const bool op_sequence = D != 128;              // the attention as single ops needs the scores and the permuted copies
+    const bool single_ropes = D % 4 != 0 || D > 256;  // the rotations and the append as single ops need a rotated k
     if (n <= pf_.rows && (keys <= pf_.keys || !op_sequence)) return GError{};
     const size_t rows = n > pf_.rows ? n : pf_.rows, kk = keys > pf_.keys ? keys : pf_.keys;
-    Prefill b;  // the old buffers are released when b replaces them: nothing of an earlier call is still queued on them
-                // only once the stream has drained
+    // The old buffers are released when b replaces them at the end; an earlier call may still be queued on them, so the
+    // stream is drained first.
+    Prefill b;
     G_TRY(dev_.gpu->check(galois_hip_synchronize(dev_.gpu->ctx())));
     const GGmlType F32 = GGmlType::F32;
     G_TRY(mk(&b.tok, GGmlType::I32, dev_, rows));
     G_TRY(mk(&b.pos, GGmlType::I32, dev_, rows));
-    for (Tensor *t : {&b.x, &b.x1, &b.q, &b.k, &b.v}) G_TRY(mk(t, F32, dev_, E, rows));
+    for (Tensor *t : {&b.x, &b.x1, &b.q, &b.k}) G_TRY(mk(t, F32, dev_, E, rows));
+    if (hp_.kv_f16) G_TRY(mk(&b.v, F32, dev_, E, rows));  // an f32 cache takes the values straight from the product
     G_TRY(mk(&b.qr, F32, dev_, D, H, rows));
-    G_TRY(mk(&b.kr, F32, dev_, D, H, rows));
+    if (single_ropes && hp_.kv_f16) G_TRY(mk(&b.kr, F32, dev_, D, H, rows));
     if (op_sequence) {
         G_TRY(mk(&b.ao, F32, dev_, E, rows));
         G_TRY(mk(&b.q3, F32, dev_, D, rows, H));
@@ -277,11 +280,11 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
         const size_t one[1] = {n}, en[2] = {E, n}, dhn[3] = {D, H, n}, dnh[3] = {D, n, H}, lnh[3] = {L, n, H};
         G_TRY(b.tok.view(0, 1, one, &tok));
         G_TRY(b.pos.view(0, 1, one, &pos));
-        for (auto pr : {std::make_pair(&b.x, &x), std::make_pair(&b.x1, &x1), std::make_pair(&b.q, &q),
-                        std::make_pair(&b.k, &k), std::make_pair(&b.v, &v)})
+        for (auto pr : {std::make_pair(&b.x, &x), std::make_pair(&b.x1, &x1), std::make_pair(&b.q, &q), std::make_pair(&b.k, &k)})
             G_TRY(pr.first->view(0, 2, en, pr.second));
+        if (hp_.kv_f16) G_TRY(b.v.view(0, 2, en, &v));
         G_TRY(b.qr.view(0, 3, dhn, &qr));
-        G_TRY(b.kr.view(0, 3, dhn, &kr));
+        if (hp_.kv_f16 && (D % 4 != 0 || D > 256)) G_TRY(b.kr.view(0, 3, dhn, &kr));
         if (D != 128) {
             G_TRY(b.ao.view(0, 2, en, &ao));
             G_TRY(b.q3.view(0, 3, dnh, &q3));
@@ -294,7 +297,7 @@ GResult LlamaDecoder::prefill(const int32_t *tokens, size_t n, int32_t n_past) {
     for (size_t i = 0; i < n; i++) positions[i] = n_past + (int32_t)i;
     G_TRY(tok.write(tokens, n * sizeof(int32_t)));
     G_TRY(pos.write(positions.data(), n * sizeof(int32_t)));
-    last_token_ = last_pos_ = -1;  // decode()'s cached inputs are not touched, but its intermediates are: see the end
+    last_token_ = last_pos_ = -1;  // the pass ends in buffers of the decode step (x_, a_, logits_): the next decode sets its inputs anew
 
     RopeCustomOption rope;
     rope.n_dims = D, rope.mode = 0, rope.n_ctx = (int32_t)C, rope.freq_base = hp_.freq_base, rope.freq_scale = hp_.freq_scale;
