@@ -445,3 +445,41 @@ def test_prefill_of_one_token_and_its_refusals(gdev):
         narrow.prefill([1, 2, 3], 0)
     assert e.value.kind == "Unimplemented"
     narrow.close()
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_prefill_at_full_width_whole_in_chunks_and_token_by_token(gdev, kv_f16):
+    """Two layers at LLaMA-7B width, 600 tokens (not a multiple of any tile): one prefill call, the same tokens as a
+    chunk of 512 and a chunk of 88 behind it, and the same tokens decoded one by one (the decode step is held to the
+    oracle above).  Chunking changes which shapes the launches take (rows per workgroup, shares of k), not what a row
+    is: logits and cache rows agree to 1e-3 between the two prefills, and to the prefill bar with the decode."""
+    rng = np.random.default_rng(61)
+    hp = dict(n_vocab=32000, n_embd=4096, n_head=32, n_layer=2, n_ff=11008, n_ctx=1024, rms_eps=1e-6, freq_base=10000.0)
+    w = _make_weights(rng, hp)
+    toks = rng.integers(0, hp["n_vocab"], 600).astype(np.int32)
+    zeros = np.zeros((hp["n_layer"], hp["n_ctx"], hp["n_embd"]), np.float16 if kv_f16 else np.float32)
+    dec = g.LlamaDecoder(gdev, kv_f16=kv_f16, **hp)
+
+    def caches():
+        return [(dec.tensor("k_cache", i).to_cpu_tensor().astype(np.float32)[:600],
+                 dec.tensor("v_cache", i).to_cpu_tensor().astype(np.float32)[:600]) for i in range(hp["n_layer"])]
+
+    _load(dec, w, zeros, zeros)
+    dec.prefill(toks, 0)
+    whole, whole_kv = dec.logits().copy(), caches()
+    assert np.all(np.isfinite(whole))
+    _load(dec, w, zeros, zeros)
+    dec.prefill(toks[:512], 0)
+    dec.prefill(toks[512:], 512)
+    _check(dec.logits(), whole, 1e-3)
+    for (k1, v1), (k2, v2) in zip(caches(), whole_kv):
+        _check(k1, k2, 1e-3)
+        _check(v1, v2, 1e-3)
+    _load(dec, w, zeros, zeros)
+    for i, t in enumerate(toks):
+        dec.decode(int(t), i, 5)
+    _check(dec.logits(), whole, PREFILL_TOL)
+    for (k1, v1), (k2, v2) in zip(caches(), whole_kv):
+        _check(k1, k2, PREFILL_TOL)
+        _check(v1, v2, PREFILL_TOL)
+    dec.close()
