@@ -791,6 +791,35 @@ int32_t launch_to_panel(galois_hip_ctx *ctx, const float *x, const float *up, _F
 
 }  // namespace
 
+namespace {
+
+// Whether one matrix against the panel is better multiplied as two shares of k, each a workgroup of 64 columns, than
+// as whole-k tiles: the cost model of gemm_launch_any (rounds of workgroups x cost of a stage x stages; a 64-column
+// stage on a full device at 0.75 of a 96-column one) plus the pass that adds the two partial results, which costs
+// about fourteen stages per 2^21 results.  Measured at M = 512 on 256 CUs: 11008 -> 4096 70.3 -> 54.8 us,
+// 4096 -> 4096 32.5 -> 30.2 us (both with the residual); the shapes the model leaves whole are slower when forced
+// into shares.  margin > 1 asks for a clearer win (where the adding pass replaces nothing the caller would launch anyway),
+// min_cost for a product large enough that the model's neglect of fixed costs does not matter.
+bool gemm_two_shares_pay(const galois_hip_ctx *ctx, int K, int N, int M, double margin = 1.0, double min_cost = 0.0) {
+    const int64_t m_tiles = (M + GM - 1) / GM, cus = ctx->n_cu > 0 ? ctx->n_cu : 256, stages = K / 64;
+    const int64_t wg96 = ((int64_t)N + 95) / 96 * m_tiles, wg48 = ((int64_t)N + 47) / 48 * m_tiles, wg64x2 = ((int64_t)N + 63) / 64 * m_tiles * 2;
+    const int64_t mn = (int64_t)M * N;
+    const double c96 = (double)((wg96 + cus - 1) / cus) * stages, c48 = 0.65 * (double)((wg48 + cus - 1) / cus) * stages;
+    const double c64x2 = 0.75 * (double)((wg64x2 + cus - 1) / cus) * (stages / 2 + 2) + 14.0 * (double)mn / (double)(1 << 21);
+    return K >= 512 && mn % 4 == 0 && margin * c64x2 < c96 && margin * c64x2 < c48 && c96 >= min_cost && c48 >= min_cost;
+}
+
+// W . panel into dst as one result (shares = 1) or as two partial results M * N floats apart (shares = 2).
+int32_t gemm_launch_shares(galois_hip_ctx *ctx, const void *W, const _Float16 *panel, float *dst, int K, int N, int M, int shares) {
+    gemm_mats mats = {};
+    mats.W[0] = (const uint8_t *)W, mats.Y[0] = dst, mats.N[0] = N;
+    if (shares == 1) return gemm_launch_any(ctx, mats, 1, panel, K, M);
+    gemm_concat(mats, 1);
+    return gemm_launch<64>(ctx, mats, panel, K, M, 2, (size_t)M * N);
+}
+
+}  // namespace
+
 extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *W, const float *X, float *Y,
                                                int32_t K, int32_t N, int32_t M) {
     GH_REQUIRE_CTX(ctx);
@@ -801,11 +830,15 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
                "mul_mat_q4_0_f32: W 2-byte, X 16-byte, Y 4-byte aligned");
     GH_BIND(ctx);
     if (gemm_panel_shape_ok(K, M) && gh_aligned(W, 16)) {
-        // fp16 copy of X, tiled for the A fragments, in the context's workspace (grown on demand)
-        const int64_t m_pad = ((int64_t)M + 15) / 16 * 16;
-        const size_t need = (size_t)m_pad * K * sizeof(_Float16);
+        // fp16 copy of X, tiled for the A fragments, in the context's workspace (grown on demand); behind it, for a
+        // matrix that is clearly better multiplied as two shares of k (512 x 11008 x 4096: 65 -> 47 us + a 5.7 us adding
+        // pass), room for the two partial results
+        const int64_t m_pad = ((int64_t)M + 15) / 16 * 16, mn = (int64_t)M * N;
+        const size_t panel_bytes = ((size_t)m_pad * K * sizeof(_Float16) + 255) & ~(size_t)255;
+        const bool shares = mn < ((int64_t)1 << 31) && gh_aligned(Y, 16) && gemm_two_shares_pay(ctx, K, N, M, 1.1, 64.0);
+        const size_t need = panel_bytes + (shares ? 2 * (size_t)mn * sizeof(float) : 0);
         if (ctx->ws_bytes < need) {
-            GH_NOT_CAPTURING(ctx, "mul_mat_q4_0_f32: growing the fp16 workspace");
+            GH_NOT_CAPTURING(ctx, "mul_mat_q4_0_f32: growing the workspace");
             // The outgrown block is kept until the context dies: work already queued, or a graph captured earlier,
             // has its address baked in.  Growing by at least half bounds what the retired blocks add up to.
             const size_t bytes = need > ctx->ws_bytes + ctx->ws_bytes / 2 ? need : ctx->ws_bytes + ctx->ws_bytes / 2;
@@ -818,10 +851,17 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *
         }
         _Float16 *Xh = (_Float16 *)ctx->ws;
         launch_to_panel(ctx, X, nullptr, Xh, K, M, false);
-        gemm_mats mats = {};
-        mats.W[0] = (const uint8_t *)W, mats.Y[0] = Y, mats.N[0] = N;
-        const int32_t st = gemm_launch_any(ctx, mats, 1, Xh, K, M);
-        if (st != GALOIS_HIP_OK) return st;
+        if (shares) {
+            float *parts = reinterpret_cast<float *>(static_cast<unsigned char *>(ctx->ws) + panel_bytes);
+            const int32_t st = gemm_launch_shares(ctx, W, Xh, parts, K, N, M, 2);
+            if (st != GALOIS_HIP_OK) return st;
+            hipLaunchKernelGGL(gemm_sum_pass, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, ctx->stream,
+                               reinterpret_cast<const float4 *>(parts), static_cast<const float4 *>(nullptr),
+                               reinterpret_cast<float4 *>(Y), mn / 4, mn / 4);
+        } else {
+            const int32_t st = gemm_launch_shares(ctx, W, Xh, Y, K, N, M, 1);
+            if (st != GALOIS_HIP_OK) return st;
+        }
     } else {
         const dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
         hipLaunchKernelGGL(gemm_q4_0_mfma_v1, grid, dim3(256), 0, ctx->stream, (const uint8_t *)W, X, Y, K, N, M);
@@ -912,33 +952,6 @@ extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel(galois_hip_ctx *ctx, const 
     GH_LAUNCH_CHECK(ctx, "mul_mat_q4_0_f16_panel launch");
 }
 
-namespace {
-
-// Whether one matrix against the panel is better multiplied as two shares of k, each a workgroup of 64 columns, than
-// as whole-k tiles: the cost model of gemm_launch_any (rounds of workgroups x cost of a stage x stages; a 64-column
-// stage on a full device at 0.75 of a 96-column one) plus the pass that adds the two partial results, which costs
-// about fourteen stages per 2^21 results.  Measured at M = 512 on 256 CUs: 11008 -> 4096 70.3 -> 54.8 us,
-// 4096 -> 4096 32.5 -> 30.2 us (both with the residual); the shapes the model leaves whole are slower when forced
-// into shares.
-bool gemm_two_shares_pay(const galois_hip_ctx *ctx, int K, int N, int M) {
-    const int64_t m_tiles = (M + GM - 1) / GM, cus = ctx->n_cu > 0 ? ctx->n_cu : 256, stages = K / 64;
-    const int64_t wg96 = ((int64_t)N + 95) / 96 * m_tiles, wg48 = ((int64_t)N + 47) / 48 * m_tiles, wg64x2 = ((int64_t)N + 63) / 64 * m_tiles * 2;
-    const int64_t mn = (int64_t)M * N;
-    const double c96 = (double)((wg96 + cus - 1) / cus) * stages, c48 = 0.65 * (double)((wg48 + cus - 1) / cus) * stages;
-    const double c64x2 = 0.75 * (double)((wg64x2 + cus - 1) / cus) * (stages / 2 + 2) + 14.0 * (double)mn / (double)(1 << 21);
-    return K >= 512 && mn % 4 == 0 && c64x2 < c96 && c64x2 < c48;
-}
-
-// W . panel into dst as one result (shares = 1) or as two partial results M * N floats apart (shares = 2).
-int32_t gemm_launch_shares(galois_hip_ctx *ctx, const void *W, const _Float16 *panel, float *dst, int K, int N, int M, int shares) {
-    gemm_mats mats = {};
-    mats.W[0] = (const uint8_t *)W, mats.Y[0] = dst, mats.N[0] = N;
-    if (shares == 1) return gemm_launch_any(ctx, mats, 1, panel, K, M);
-    gemm_concat(mats, 1);
-    return gemm_launch<64>(ctx, mats, panel, K, M, 2, (size_t)M * N);
-}
-
-}  // namespace
 
 // One matrix against the panel with a residual added, and the k-split shape for matrices too narrow to fill the device.
 extern "C" int32_t galois_hip_mul_mat_q4_0_f16_panel_add(galois_hip_ctx *ctx, const void *W, const void *panel, const float *residual,
