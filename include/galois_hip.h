@@ -194,7 +194,11 @@ int32_t galois_hip_dequantize_mul_mat_vec_q4_0_group(galois_hip_ctx *ctx, const 
  * matmul.cu:133-174,452-504) with one call: Y[m*N + n] = sum_k deq(W)[n,k] * X[m*K + k]
  * (output layout of matmul.cu:359).  W tiles are dequantised to fp16 in LDS, X is
  * rounded to fp16, products accumulate in f32 on MFMA.  K % 32 == 0.  No Q8_1
- * scratch and no K padding (src/cuda.rs:1040-1068) are needed. */
+ * scratch and no K padding (src/cuda.rs:1040-1068) are needed.  The fp16 copy of X lives in a workspace the context
+ * owns and grows on demand (the call allocates when a larger one is needed; refused during a graph capture).  A large
+ * product whose N leaves compute units idle (512 x 11008 x 4096 on 256 CUs) is computed as two shares of k that a
+ * second launch adds: the f32 sums over k are then two chains instead of one, for the same operands on the same
+ * device always the same way. */
 int32_t galois_hip_mul_mat_q4_0_f32(galois_hip_ctx *ctx, const void *W, const float *X, float *Y,
                                     int32_t K, int32_t N, int32_t M);
 
