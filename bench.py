@@ -330,23 +330,29 @@ def decode_step_bench(dev, reps, with_graph=True, prefill_only=False):
         return {"max_rel": float(np.max(np.abs(a - b)) / np.max(np.abs(b))),
                 "l2_rel": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
 
-    def prefill(dec, n_tok=512):
+    def prefill(dec, n_tok=512, compare=True):
         """n_tok tokens from an empty context in one pass (LlamaDecoder.prefill: the Q4_0 products through the prefill
         matmul on fp16 panels) against the same tokens decoded one by one on the same decoder."""
         hp = dec.hp
         e, f = hp["n_embd"], hp["n_ff"]
         toks = np.random.default_rng(11).integers(0, hp["n_vocab"], n_tok).astype(np.int32)
-        t_dec = time.time()
-        for i, t in enumerate(toks):
-            dec.decode(int(t), i, 5)
-        one_by_one = dec.logits().astype(np.float64)     # (the download waits for the stream)
-        ms_one_by_one = (time.time() - t_dec) * 1e3
+        if compare:
+            t_dec = time.time()
+            for i, t in enumerate(toks):
+                dec.decode(int(t), i, 5)
+            one_by_one = dec.logits().astype(np.float64)     # (the download waits for the stream)
+            ms_one_by_one = (time.time() - t_dec) * 1e3
         dec.prefill(toks, 0)
         got = dec.logits().astype(np.float64)
         dec.time_prefill(toks, 0, 4)
         ms = min(dec.time_prefill(toks, 0, 4) for _ in range(3)) / 4
         q4_flop = 2.0 * n_tok * hp["n_layer"] * (4 * e * e + 3 * e * f)
         attn_flop = 2.0 * 2 * n_tok * n_tok * e * hp["n_layer"]     # scores and out over all n_tok keys (the masked half too)
+        if not compare:
+            return {"tokens": n_tok, "library_calls": dec.ops_per_prefill(), "ms": round(ms, 3), "tokens_per_s": round(n_tok / ms * 1e3, 0),
+                    "q4_0_flop_over_the_whole_pass_TFLOPs": round(q4_flop / ms / 1e9, 1),
+                    "q4_0_flop_over_the_whole_pass_mfma_frac": round(q4_flop / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                    "logits_finite": bool(np.all(np.isfinite(got)))}
         return {"tokens": n_tok, "library_calls": dec.ops_per_prefill(), "ms": round(ms, 3), "tokens_per_s": round(n_tok / ms * 1e3, 0),
                 "q4_0_flop_over_the_whole_pass_TFLOPs": round(q4_flop / ms / 1e9, 1),
                 "q4_0_flop_over_the_whole_pass_mfma_frac": round(q4_flop / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
@@ -390,6 +396,7 @@ def decode_step_bench(dev, reps, with_graph=True, prefill_only=False):
     res["logits_within_1e-4"] = bool(all(v["max_rel"] < 1e-4 and v["l2_rel"] < 1e-4
                                          for v in res["logits_vs_one_kernel_per_op"].values()))
     res["prefill_512_tokens"] = prefill(dec)
+    res["prefill_2048_tokens"] = prefill(dec, 2048, compare=False)   # a whole context in one pass
     dec.close()
     # the same step with the caches kept [n_head][n_ctx][head_dim]: a head's keys contiguous (same weights, same cache
     # contents: the logits are compared with the one-kernel-per-op plan of the [n_ctx][n_embd] decoder above)
